@@ -1,0 +1,259 @@
+// C ABI of libpkh3attn.so: argument validation (host only, before any HIP call), workspace
+// planning, and the sequence of launches that makes up one attention call.
+#include "../../include/pkh3_attn.h"
+
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "pkh3_common.h"
+#include "pkh3_internal.h"
+
+using namespace pkh3;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+bool misaligned16(const void* p) { return ((uintptr_t)p & 15u) != 0; }
+
+int check_tensor(const char* name, const void* ptr, int64_t sb, int64_t ss, int64_t sh, int B, int H) {
+  if (!ptr) return fail(PKH3_ENULL, "%s is NULL", name);
+  if (misaligned16(ptr)) return fail(PKH3_EALIGN, "%s is not 16-byte aligned", name);
+  if (sb < 0 || ss < 0 || sh < 0) return fail(PKH3_ESTRIDE, "%s: negative stride", name);
+  if ((ss % 8) || (sh % 8) || (B > 1 && (sb % 8)))
+    return fail(PKH3_ESTRIDE, "%s: strides must be multiples of 8 elements (16-byte rows), got (%lld, %lld, %lld)", name,
+                (long long)sb, (long long)ss, (long long)sh);
+  if (H > 1 && sh == 0) return fail(PKH3_ESTRIDE, "%s: head stride is 0", name);
+  return PKH3_OK;
+}
+
+// Validation shared by pkh3_workspace_bytes (shapes/options only) and pkh3_attn_fwd (everything).
+int validate(const pkh3_attn_args* a, bool pointers) {
+  if (!a) return fail(PKH3_ENULL, "args is NULL");
+  if (a->D != kD) return fail(PKH3_EHEADDIM, "head dim must be 128, got %d", a->D);
+  if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Sk < 1) return fail(PKH3_ESHAPE, "B, H, Sq, Sk must be >= 1");
+  if (a->B > 65535 || a->H > 65535) return fail(PKH3_ESHAPE, "B and H must be <= 65535");
+  if (a->Sq > (1 << 24) || a->Sk > (1 << 24)) return fail(PKH3_ESHAPE, "Sq and Sk must be <= 2^24");
+  if (a->flags & ~(uint32_t)PKH3_FLAG_FP8_QK) return fail(PKH3_EARG, "unknown flag bits 0x%x", a->flags);
+  if (a->rope_mode < PKH3_ROPE_NONE || a->rope_mode > PKH3_ROPE_HALF) return fail(PKH3_EARG, "bad rope_mode %d", a->rope_mode);
+  if (!(a->softmax_scale == a->softmax_scale) || isinf(a->softmax_scale)) return fail(PKH3_EARG, "softmax_scale is not finite");
+  if ((a->q_norm_w || a->k_norm_w) && !(a->norm_eps >= 0.f)) return fail(PKH3_EARG, "norm_eps must be >= 0");
+  if ((a->blk_row_ptr == nullptr) != (a->blk_col_idx == nullptr))
+    return fail(PKH3_ENULL, "blk_row_ptr and blk_col_idx must be given together");
+  if (a->blk_row_ptr && a->key_mask) return fail(PKH3_EUNSUPPORTED, "block-sparse map together with a key mask is not supported");
+  if (!pointers) return PKH3_OK;
+  int rc;
+  if ((rc = check_tensor("q", a->q, a->q_sb, a->q_ss, a->q_sh, a->B, a->H))) return rc;
+  if ((rc = check_tensor("k", a->k, a->k_sb, a->k_ss, a->k_sh, a->B, a->H))) return rc;
+  if ((rc = check_tensor("v", a->v, a->v_sb, a->v_ss, a->v_sh, a->B, a->H))) return rc;
+  if ((rc = check_tensor("o", a->o, a->o_sb, a->o_ss, a->o_sh, a->B, a->H))) return rc;
+  if (a->rope_mode != PKH3_ROPE_NONE) {
+    if (!a->q_rope_cos || !a->q_rope_sin || !a->k_rope_cos || !a->k_rope_sin)
+      return fail(PKH3_ENULL, "rope_mode set but a cos/sin table is NULL");
+    if (misaligned16(a->q_rope_cos) || misaligned16(a->q_rope_sin) || misaligned16(a->k_rope_cos) || misaligned16(a->k_rope_sin))
+      return fail(PKH3_EALIGN, "rope tables must be 16-byte aligned");
+  }
+  if ((a->q_norm_w && misaligned16(a->q_norm_w)) || (a->k_norm_w && misaligned16(a->k_norm_w)))
+    return fail(PKH3_EALIGN, "norm weights must be 16-byte aligned");
+  if (!a->workspace) return fail(PKH3_EWORKSPACE, "workspace is NULL");
+  if ((uintptr_t)a->workspace & 255u) return fail(PKH3_EWORKSPACE, "workspace is not 256-byte aligned");
+  return PKH3_OK;
+}
+
+WsPlan plan(const pkh3_attn_args* a) {
+  WsPlan w{};
+  const bool fp8 = a->flags & PKH3_FLAG_FP8_QK;
+  w.nQ64 = (int)align_up((size_t)(a->Sq + 63) / 64, 4);
+  w.nKt = (a->Sk + 63) / 64;
+  w.kvTileBytes = (fp8 ? kK8TileBytes : kKTileBytes) + kVTileBytes;
+  w.qBlkBytes = fp8 ? 2 * kQ8BlkBytes : 2 * kQBlkBytes;
+  const size_t bh = (size_t)a->B * a->H;
+  size_t off = 0;
+  w.q_off = off;      off = align_up(off + bh * w.nQ64 * w.qBlkBytes, 256);
+  w.kv_off = off;     off = align_up(off + bh * w.nKt * (size_t)w.kvTileBytes, 256);
+  w.qscale_off = off; if (fp8) off = align_up(off + bh * w.nQ64 * sizeof(float), 256);
+  w.kscale_off = off; if (fp8) off = align_up(off + bh * w.nKt * sizeof(float), 256);
+  w.cnt_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * sizeof(int), 256);
+  w.idx_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * a->Sk * sizeof(int), 256);
+  w.total = off;
+  return w;
+}
+
+struct Launch {
+  WsPlan w;
+  QkPrologueParams qp, kp;
+  VPrologueParams vp;
+  FwdParams f;
+  int* cnt;
+  int* idx;
+};
+
+void build(const pkh3_attn_args* a, Launch& L) {
+  const bool fp8 = a->flags & PKH3_FLAG_FP8_QK;
+  L.w = plan(a);
+  char* ws = (char*)a->workspace;
+  L.cnt = a->key_mask ? (int*)(ws + L.w.cnt_off) : nullptr;
+  L.idx = a->key_mask ? (int*)(ws + L.w.idx_off) : nullptr;
+  const int kBytes = fp8 ? kK8TileBytes : kKTileBytes;
+
+  QkPrologueParams& q = L.qp;
+  q = QkPrologueParams{};
+  q.x = a->q; q.sb = a->q_sb; q.ss = a->q_ss; q.sh = a->q_sh;
+  q.B = a->B; q.H = a->H; q.S = a->Sq; q.nBlk64 = L.w.nQ64;
+  q.norm_w = a->q_norm_w; q.eps = a->norm_eps; q.rope_mode = a->rope_mode;
+  q.cos_t = a->q_rope_cos; q.sin_t = a->q_rope_sin;
+  q.out = ws + L.w.q_off; q.out_bh_stride = (int64_t)L.w.nQ64 * L.w.qBlkBytes; q.out_blk_stride = L.w.qBlkBytes;
+  q.scale_out = fp8 ? (float*)(ws + L.w.qscale_off) : nullptr; q.fp8 = fp8;
+
+  QkPrologueParams& k = L.kp;
+  k = QkPrologueParams{};
+  k.x = a->k; k.sb = a->k_sb; k.ss = a->k_ss; k.sh = a->k_sh;
+  k.B = a->B; k.H = a->H; k.S = a->Sk; k.nBlk64 = L.w.nKt;
+  k.norm_w = a->k_norm_w; k.eps = a->norm_eps; k.rope_mode = a->rope_mode;
+  k.cos_t = a->k_rope_cos; k.sin_t = a->k_rope_sin;
+  k.gather_idx = L.idx; k.row_cnt = L.cnt;
+  k.out = ws + L.w.kv_off; k.out_bh_stride = (int64_t)L.w.nKt * L.w.kvTileBytes; k.out_blk_stride = L.w.kvTileBytes;
+  k.scale_out = fp8 ? (float*)(ws + L.w.kscale_off) : nullptr; k.fp8 = fp8;
+
+  VPrologueParams& v = L.vp;
+  v = VPrologueParams{};
+  v.v = a->v; v.sb = a->v_sb; v.ss = a->v_ss; v.sh = a->v_sh;
+  v.B = a->B; v.H = a->H; v.S = a->Sk; v.nKt = L.w.nKt;
+  v.gather_idx = L.idx; v.row_cnt = L.cnt;
+  v.out = ws + L.w.kv_off + kBytes; v.out_bh_stride = k.out_bh_stride; v.out_tile_stride = L.w.kvTileBytes;
+
+  FwdParams& f = L.f;
+  f = FwdParams{};
+  f.qp = ws + L.w.q_off; f.q_bh_stride = q.out_bh_stride; f.q_blk_stride = L.w.qBlkBytes;
+  f.kv = ws + L.w.kv_off; f.kv_bh_stride = k.out_bh_stride; f.kv_tile_stride = L.w.kvTileBytes;
+  f.row_cnt = L.cnt;
+  f.o = a->o; f.o_sb = a->o_sb; f.o_ss = a->o_ss; f.o_sh = a->o_sh;
+  f.B = a->B; f.H = a->H; f.Sq = a->Sq; f.Sk = a->Sk; f.nQ64 = L.w.nQ64; f.nKt = L.w.nKt;
+  const float scale = a->softmax_scale > 0.f ? a->softmax_scale : 1.0f / sqrtf((float)kD);
+  f.c = scale * kLog2e;
+  f.blk_row_ptr = a->blk_row_ptr; f.blk_col_idx = a->blk_col_idx;
+  f.qscale = q.scale_out; f.kscale = k.scale_out; f.fp8 = fp8;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(PKH3_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int run_prologue(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
+  hipError_t e;
+  if (a->key_mask) {
+    if ((e = launch_mask_compact(a->key_mask, a->B, a->Sk, L.idx, L.cnt, st)) != hipSuccess) return hip_fail(e, "mask_compact");
+  }
+  if ((e = launch_qk_prologue(L.qp, st)) != hipSuccess) return hip_fail(e, "q prologue");
+  if ((e = launch_qk_prologue(L.kp, st)) != hipSuccess) return hip_fail(e, "k prologue");
+  if ((e = launch_v_prologue(L.vp, st)) != hipSuccess) return hip_fail(e, "v prologue");
+  return PKH3_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pkh3_version(void) { return PKH3_VERSION; }
+
+const char* pkh3_last_error(void) { return g_err; }
+
+const char* pkh3_strerror(int code) {
+  switch (code) {
+    case PKH3_OK: return "ok";
+    case PKH3_ENULL: return "required pointer is NULL";
+    case PKH3_ESHAPE: return "shape out of range";
+    case PKH3_EHEADDIM: return "head dim must be 128";
+    case PKH3_ESTRIDE: return "bad stride";
+    case PKH3_EALIGN: return "pointer not 16-byte aligned";
+    case PKH3_EWORKSPACE: return "workspace missing, misaligned or too small";
+    case PKH3_EUNSUPPORTED: return "unsupported combination of options";
+    case PKH3_EHIP: return "HIP runtime error";
+    case PKH3_EARG: return "invalid argument";
+    default: return "unknown error code";
+  }
+}
+
+size_t pkh3_workspace_bytes(const pkh3_attn_args* a) {
+  if (validate(a, false) != PKH3_OK) return 0;
+  return plan(a).total;
+}
+
+int pkh3_attn_fwd(const pkh3_attn_args* a, void* stream) {
+  int rc = validate(a, true);
+  if (rc) return rc;
+  Launch L;
+  build(a, L);
+  if (a->workspace_bytes < L.w.total)
+    return fail(PKH3_EWORKSPACE, "workspace too small: %zu < %zu bytes", a->workspace_bytes, L.w.total);
+  hipStream_t st = (hipStream_t)stream;
+  if ((rc = run_prologue(a, L, st))) return rc;
+  hipError_t e = launch_attn_fwd(L.f, st);
+  if (e != hipSuccess) return hip_fail(e, "attn_fwd");
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
+int pkh3_attn_time_kernel(const pkh3_attn_args* a, void* stream, int iters, float* ms_out) {
+  if (!ms_out) return fail(PKH3_ENULL, "ms_out is NULL");
+  if (iters < 1) return fail(PKH3_EARG, "iters must be >= 1");
+  int rc = validate(a, true);
+  if (rc) return rc;
+  Launch L;
+  build(a, L);
+  if (a->workspace_bytes < L.w.total)
+    return fail(PKH3_EWORKSPACE, "workspace too small: %zu < %zu bytes", a->workspace_bytes, L.w.total);
+  hipStream_t st = (hipStream_t)stream;
+  if ((rc = run_prologue(a, L, st))) return rc;
+  hipError_t e;
+  if ((e = launch_attn_fwd(L.f, st)) != hipSuccess) return hip_fail(e, "attn_fwd");  // warm
+  hipEvent_t e0, e1;
+  if ((e = hipEventCreate(&e0)) != hipSuccess) return hip_fail(e, "hipEventCreate");
+  if ((e = hipEventCreate(&e1)) != hipSuccess) { hipEventDestroy(e0); return hip_fail(e, "hipEventCreate"); }
+  hipEventRecord(e0, st);
+  for (int i = 0; i < iters; ++i) {
+    if ((e = launch_attn_fwd(L.f, st)) != hipSuccess) break;
+  }
+  hipEventRecord(e1, st);
+  hipError_t es = hipEventSynchronize(e1);
+  float ms = 0.f;
+  if (e == hipSuccess && es == hipSuccess) hipEventElapsedTime(&ms, e0, e1);
+  hipEventDestroy(e0);
+  hipEventDestroy(e1);
+  if (e != hipSuccess) return hip_fail(e, "attn_fwd");
+  if (es != hipSuccess) return hip_fail(es, "hipEventSynchronize");
+  *ms_out = ms / iters;
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
+int pkh3_rope_tables(const double* position_ids, int32_t S, const int32_t axis_dims[3], double theta, float* cos_out,
+                     float* sin_out, void* stream) {
+  if (!position_ids || !axis_dims || !cos_out || !sin_out) return fail(PKH3_ENULL, "rope_tables: NULL argument");
+  if (S < 1) return fail(PKH3_ESHAPE, "rope_tables: S must be >= 1");
+  int sum = 0;
+  for (int i = 0; i < 3; ++i) {
+    if (axis_dims[i] < 0 || (axis_dims[i] & 1)) return fail(PKH3_EARG, "rope_tables: axis dims must be even and >= 0");
+    sum += axis_dims[i];
+  }
+  if (sum != kD) return fail(PKH3_EARG, "rope_tables: axis dims must sum to 128, got %d", sum);
+  if (!(theta > 1.0)) return fail(PKH3_EARG, "rope_tables: theta must be > 1");
+  hipError_t e = launch_rope_tables(position_ids, S, axis_dims, theta, cos_out, sin_out, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "rope_tables");
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
+}  // extern "C"

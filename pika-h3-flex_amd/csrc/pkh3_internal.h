@@ -1,0 +1,76 @@
+// Host-side structures shared by the C-ABI translation unit and the kernel launchers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace pkh3 {
+
+// Where each intermediate lives inside the caller's workspace (byte offsets, 256-aligned).
+struct WsPlan {
+  int nQ64;      // 64-query blocks, padded to a multiple of 4 (one workgroup = 4 waves x 64 queries)
+  int nKt;       // 64-key tiles
+  int kvTileBytes;  // bytes of one [K tile | V tile] record
+  int qBlkBytes;    // bytes of one 64-query block of Q images
+  size_t q_off, kv_off, qscale_off, kscale_off, cnt_off, idx_off, total;
+};
+
+// One side (Q or K) of the normalise + rotate + lay-out pass.
+struct QkPrologueParams {
+  const void* x;            // bf16 [B,S,H,D] strided
+  int64_t sb, ss, sh;
+  int B, H, S;
+  int nBlk64;               // 64-row blocks to write (>= ceil(S/64); rows past the end are zero)
+  const float* norm_w;      // [D] or null
+  float eps;
+  int rope_mode;
+  const float* cos_t;       // [S, D/2] or null
+  const float* sin_t;
+  const int* gather_idx;    // [B, S] compacted row -> source row, or null
+  const int* row_cnt;       // [B] rows that exist after compaction, or null (= S)
+  char* out;                // images
+  int64_t out_bh_stride;    // bytes between consecutive (b,h)
+  int out_blk_stride;       // bytes between consecutive 64-row blocks
+  float* scale_out;         // fp8: [B*H, nBlk64] dequantisation scales, else null
+  int fp8;
+};
+
+struct VPrologueParams {
+  const void* v;
+  int64_t sb, ss, sh;
+  int B, H, S, nKt;
+  const int* gather_idx;
+  const int* row_cnt;
+  char* out;                // points at the V part of tile 0
+  int64_t out_bh_stride;
+  int out_tile_stride;
+};
+
+struct FwdParams {
+  const char* qp;           // Q images
+  int64_t q_bh_stride;      // bytes
+  int q_blk_stride;         // bytes per 64-query block
+  const char* kv;           // [K tile | V tile] records
+  int64_t kv_bh_stride;
+  int kv_tile_stride;
+  const int* row_cnt;       // [B] valid keys after compaction, or null (= Sk)
+  void* o;
+  int64_t o_sb, o_ss, o_sh;
+  int B, H, Sq, Sk;
+  int nQ64, nKt;
+  float c;                  // softmax_scale * log2(e)
+  const int* blk_row_ptr;
+  const int* blk_col_idx;
+  const float* qscale;      // [B*H, nQ64]
+  const float* kscale;      // [B*H, nKt]
+  int fp8;
+};
+
+hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int* cnt, hipStream_t st);
+hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st);
+hipError_t launch_v_prologue(const VPrologueParams& p, hipStream_t st);
+hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st);
+hipError_t launch_rope_tables(const double* pos, int S, const int* axis_dims, double theta, float* cos_out,
+                              float* sin_out, hipStream_t st);
+
+}  // namespace pkh3

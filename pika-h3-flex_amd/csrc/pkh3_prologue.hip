@@ -1,0 +1,252 @@
+// Prologue kernels: everything that touches each Q/K/V row exactly once before the S x S work.
+//   - key-mask compaction (prefix sum of the padding mask -> list of valid key rows)
+//   - QK-RMSNorm + rotary embedding (+ optional fp8 e4m3 quantisation with per-64-row absmax scales),
+//     written as MFMA operand images
+//   - V re-laid out as the A-operand images of O^T = V^T P^T
+//   - rotary cos/sin tables from the float64 position grid
+// All of it is HBM-bound streaming work (a few hundred MB per layer call against ~29 TFLOP of
+// attention), so the kernels are plain coalesced-store loops with no LDS staging.
+#include "pkh3_common.h"
+#include "pkh3_internal.h"
+
+namespace pkh3 {
+
+// ------------------------------------------------------------------------------------------------
+// Key-mask compaction: idx[b][slot] = key index of the slot-th valid key, cnt[b] = number of valid keys.
+// One workgroup of 1024 threads per batch walks the mask in chunks, carrying the running count.
+__global__ __launch_bounds__(1024) void mask_compact_kernel(const uint8_t* __restrict__ mask, int Sk,
+                                                            int* __restrict__ idx, int* __restrict__ cnt) {
+  __shared__ int wave_tot[16];
+  __shared__ int carry;
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint8_t* m = mask + (int64_t)b * Sk;
+  int* out = idx + (int64_t)b * Sk;
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int base = 0; base < Sk; base += 1024) {
+    const int key = base + tid;
+    const bool on = key < Sk && m[key] != 0;
+    const unsigned long long bal = __ballot(on);
+    const int before = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_tot[wave] = __popcll(bal);
+    __syncthreads();
+    int off = carry;
+    for (int w = 0; w < wave; ++w) off += wave_tot[w];
+    if (on) out[off + before] = key;
+    __syncthreads();
+    if (tid == 0) {
+      int t = carry;
+      for (int w = 0; w < 16; ++w) t += wave_tot[w];
+      carry = t;
+    }
+    __syncthreads();
+  }
+  if (tid == 0) cnt[b] = carry;
+}
+
+hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int* cnt, hipStream_t st) {
+  hipLaunchKernelGGL(mask_compact_kernel, dim3(B), dim3(1024), 0, st, mask, Sk, idx, cnt);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------------
+// RMSNorm + RoPE (+ fp8 quantisation) of Q or K rows into operand images.
+// One wave owns one 64-row block of one (batch, head): lane (r = l%32, hh = l/32) holds, for the
+// two 32-row halves `sub`, the 64 elements d = 16*ks + 8*hh + j of row 32*sub + r -- exactly the
+// elements its lane carries in the MFMA images, so norm, rotation and the store need one
+// cross-lane exchange only (the sum of squares with lane l^32).
+template <bool FP8>
+__global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int blk = blockIdx.x * 4 + wave;
+  if (blk >= p.nBlk64) return;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int r = lane & 31, hh = lane >> 5;
+  const int rows = p.row_cnt ? p.row_cnt[b] : p.S;
+  const __bf16* xb = (const __bf16*)p.x + (int64_t)b * p.sb + (int64_t)h * p.sh;
+
+  float x[2][64];
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub) {
+    const int row = blk * 64 + sub * 32 + r;
+    const bool valid = row < rows;
+    int src = 0;
+    if (valid) src = p.gather_idx ? p.gather_idx[(int64_t)b * p.S + row] : row;
+    const __bf16* xr = xb + (int64_t)src * p.ss;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      bf16x8 t = {};
+      if (valid) t = *(const bf16x8*)(xr + 16 * ks + 8 * hh);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[sub][ks * 8 + j] = (float)t[j];
+    }
+    if (p.norm_w) {
+      float ssq = 0.f;
+#pragma unroll
+      for (int i = 0; i < 64; ++i) ssq += x[sub][i] * x[sub][i];
+      ssq += xhalf(ssq);
+      const float rs = rsqrtf(ssq * (1.0f / kD) + p.eps);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const f32x4 w0 = *(const f32x4*)(p.norm_w + 16 * ks + 8 * hh);
+        const f32x4 w1 = *(const f32x4*)(p.norm_w + 16 * ks + 8 * hh + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          x[sub][ks * 8 + j] *= rs * w0[j];
+          x[sub][ks * 8 + 4 + j] *= rs * w1[j];
+        }
+      }
+    }
+    if (p.rope_mode == 1 && valid) {
+      // interleaved pairs (2i, 2i+1): pair index 8*ks + 4*hh + jj for this lane's elements 2jj, 2jj+1
+      const float* ct = p.cos_t + (int64_t)src * (kD / 2);
+      const float* st = p.sin_t + (int64_t)src * (kD / 2);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const f32x4 c = *(const f32x4*)(ct + 8 * ks + 4 * hh);
+        const f32x4 s = *(const f32x4*)(st + 8 * ks + 4 * hh);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const float a0 = x[sub][ks * 8 + 2 * jj], a1 = x[sub][ks * 8 + 2 * jj + 1];
+          x[sub][ks * 8 + 2 * jj] = a0 * c[jj] - a1 * s[jj];
+          x[sub][ks * 8 + 2 * jj + 1] = a1 * c[jj] + a0 * s[jj];
+        }
+      }
+    } else if (p.rope_mode == 2 && valid) {
+      // half-split pairs (i, i + 64): element d < 64 of this lane sits at ks < 4, its partner at ks + 4
+      const float* ct = p.cos_t + (int64_t)src * (kD / 2);
+      const float* st = p.sin_t + (int64_t)src * (kD / 2);
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+        for (int q4 = 0; q4 < 2; ++q4) {
+          const f32x4 c = *(const f32x4*)(ct + 16 * ks + 8 * hh + 4 * q4);
+          const f32x4 s = *(const f32x4*)(st + 16 * ks + 8 * hh + 4 * q4);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float lo = x[sub][ks * 8 + 4 * q4 + j], hi = x[sub][(ks + 4) * 8 + 4 * q4 + j];
+            x[sub][ks * 8 + 4 * q4 + j] = lo * c[j] - hi * s[j];
+            x[sub][(ks + 4) * 8 + 4 * q4 + j] = hi * c[j] + lo * s[j];
+          }
+        }
+      }
+    }
+  }
+
+  char* ob = p.out + (int64_t)(b * p.H + h) * p.out_bh_stride + (int64_t)blk * p.out_blk_stride;
+  if constexpr (!FP8) {
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        bf16x8 t;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[sub][ks * 8 + j];
+        *(bf16x8*)(ob + ((sub * 8 + ks) * 64 + lane) * 16) = t;
+      }
+  } else {
+    float amax = 0.f;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int i = 0; i < 64; ++i) amax = fmaxf(amax, fabsf(x[sub][i]));
+    amax = wave_max(amax);
+    const float scale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
+    const float inv = 1.0f / scale;
+    if (lane == 0) p.scale_out[(int64_t)(b * p.H + h) * p.nBlk64 + blk] = scale;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        i32x4 t;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const float* e = &x[sub][c * 16 + w * 4];
+          int v = 0;
+          v = __builtin_amdgcn_cvt_pk_fp8_f32(e[0] * inv, e[1] * inv, v, false);
+          v = __builtin_amdgcn_cvt_pk_fp8_f32(e[2] * inv, e[3] * inv, v, true);
+          t[w] = v;
+        }
+        *(i32x4*)(ob + ((sub * 4 + c) * 64 + lane) * 16) = t;
+      }
+  }
+}
+
+hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st) {
+  dim3 grid((p.nBlk64 + 3) / 4, p.H, p.B);
+  if (p.fp8)
+    hipLaunchKernelGGL(qk_prologue_kernel<true>, grid, dim3(256), 0, st, p);
+  else
+    hipLaunchKernelGGL(qk_prologue_kernel<false>, grid, dim3(256), 0, st, p);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------------
+// V rows -> A-operand images of O^T = V^T P^T.  One wave per 64-key tile of one (batch, head).
+// Lane (r, hh) of image (kb, b2, db) needs V[key(kb,b2,hh,j)][32*db + r] for j = 0..7: eight rows at
+// one column.  Reads are 2-byte gathers (64 B contiguous per half-wave, served from L1/L2); the
+// stores are full 1 KiB lines.
+__global__ __launch_bounds__(256) void v_prologue_kernel(VPrologueParams p) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= p.nKt) return;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int r = lane & 31, hh = lane >> 5;
+  const int rows = p.row_cnt ? p.row_cnt[b] : p.S;
+  const __bf16* vb = (const __bf16*)p.v + (int64_t)b * p.sb + (int64_t)h * p.sh;
+  char* ob = p.out + (int64_t)(b * p.H + h) * p.out_bh_stride + (int64_t)t * p.out_tile_stride;
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int b2 = 0; b2 < 2; ++b2) {
+      bf16x8 img[4];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int row = t * 64 + kb * 32 + 8 * (2 * b2 + j / 4) + 4 * hh + (j % 4);
+        const bool valid = row < rows;
+        int src = 0;
+        if (valid) src = p.gather_idx ? p.gather_idx[(int64_t)b * p.S + row] : row;
+        const __bf16* vr = vb + (int64_t)src * p.ss + r;
+#pragma unroll
+        for (int db = 0; db < 4; ++db) img[db][j] = valid ? vr[32 * db] : (__bf16)0.0f;
+      }
+#pragma unroll
+      for (int db = 0; db < 4; ++db) *(bf16x8*)(ob + (((kb * 2 + b2) * 4 + db) * 64 + lane) * 16) = img[db];
+    }
+}
+
+hipError_t launch_v_prologue(const VPrologueParams& p, hipStream_t st) {
+  dim3 grid((p.nKt + 3) / 4, p.H, p.B);
+  hipLaunchKernelGGL(v_prologue_kernel, grid, dim3(256), 0, st, p);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------------
+// cos/sin tables from the [S,3] float64 position grid.  Pair p of the D/2 = 64 pairs belongs to the
+// axis whose slice contains it; inside its slice of n = axis_dims[a]/2 pairs, pair i rotates by
+// pos[a] * theta^(-2i / axis_dims[a]).  Computed in float64, stored fp32.
+__global__ void rope_tables_kernel(const double* __restrict__ pos, int S, int d0, int d1, int d2, double log_theta,
+                                   float* __restrict__ cos_out, float* __restrict__ sin_out) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (int64_t)S * (kD / 2)) return;
+  const int s = (int)(gid / (kD / 2)), pr = (int)(gid % (kD / 2));
+  int a, i, dim;
+  if (pr < d0 / 2) { a = 0; i = pr; dim = d0; }
+  else if (pr < (d0 + d1) / 2) { a = 1; i = pr - d0 / 2; dim = d1; }
+  else { a = 2; i = pr - (d0 + d1) / 2; dim = d2; }
+  const double freq = exp(-log_theta * (2.0 * i) / (double)dim);
+  const double ang = pos[(int64_t)s * 3 + a] * freq;
+  cos_out[gid] = (float)cos(ang);
+  sin_out[gid] = (float)sin(ang);
+}
+
+hipError_t launch_rope_tables(const double* pos, int S, const int* axis_dims, double theta, float* cos_out,
+                              float* sin_out, hipStream_t st) {
+  const int64_t n = (int64_t)S * (kD / 2);
+  hipLaunchKernelGGL(rope_tables_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, pos, S, axis_dims[0],
+                     axis_dims[1], axis_dims[2], log(theta), cos_out, sin_out);
+  return hipGetLastError();
+}
+
+}  // namespace pkh3

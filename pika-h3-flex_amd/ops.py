@@ -1,0 +1,180 @@
+"""Tensor-level front end of the C ABI: takes torch tensors (device memory + strides), fills
+``pkh3_attn_args`` and enqueues the call on torch's current HIP stream.  PyTorch is used here for
+memory and streams only; all arithmetic happens in libpkh3attn.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+HEAD_DIM = 128
+
+
+@dataclass
+class BlockMask:
+    """64x64-tile block-sparse map in CSR form (int32, on the device), shared by batches and heads."""
+
+    row_ptr: torch.Tensor  # [ceil(Sq/64)+1]
+    col_idx: torch.Tensor  # [nnz]
+
+    @staticmethod
+    def from_dense(tile_map: torch.Tensor, device=None) -> "BlockMask":
+        """``tile_map``: bool [ceil(Sq/64), ceil(Sk/64)], True = compute that tile."""
+        tm = tile_map.to("cpu", torch.bool)
+        counts = tm.sum(dim=1, dtype=torch.int64)
+        row_ptr = torch.zeros(tm.shape[0] + 1, dtype=torch.int32)
+        row_ptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+        col_idx = tm.nonzero(as_tuple=False)[:, 1].to(torch.int32).contiguous()
+        if col_idx.numel() == 0:
+            col_idx = torch.zeros(1, dtype=torch.int32)
+        dev = device if device is not None else tile_map.device
+        return BlockMask(row_ptr.to(dev), col_idx.to(dev))
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _check_bshd(name: str, t: torch.Tensor) -> None:
+    if t.dim() != 4:
+        raise ValueError(f"{name} must be [B, S, H, D], got shape {tuple(t.shape)}")
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
+    if t.stride(3) != 1:
+        raise ValueError(f"{name}: head-dim stride must be 1, got {t.stride(3)}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live in device memory (got {t.device}); the HIP library is the only compute path")
+
+
+def _f32(name: str, t: Optional[torch.Tensor], shape) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must be contiguous float32 {tuple(shape)}, got {t.dtype} {tuple(t.shape)}")
+    return t
+
+
+def fill_args(
+    q, k, v, out, *, q_norm_weight=None, k_norm_weight=None, norm_eps=1e-6, rope_q=None, rope_k=None,
+    rope_mode=_lib.ROPE_NONE, key_mask=None, block_mask: Optional[BlockMask] = None, fp8_qk=False,
+    softmax_scale: Optional[float] = None,
+) -> Tuple[_lib.AttnArgs, list]:
+    """Build ``pkh3_attn_args`` for these tensors.  Returns (args, keep_alive)."""
+    for n, t in (("q", q), ("k", k), ("v", v), ("out", out)):
+        _check_bshd(n, t)
+    B, Sq, H, D = q.shape
+    Sk = k.shape[1]
+    if tuple(k.shape) != (B, Sk, H, D) or tuple(v.shape) != (B, Sk, H, D):
+        raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
+    if tuple(out.shape) != (B, Sq, H, D):
+        raise ValueError(f"out shape {tuple(out.shape)} != {(B, Sq, H, D)}")
+    keep = [q, k, v, out]
+    a = _lib.AttnArgs()
+    a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.q_sb, a.q_ss, a.q_sh = q.stride(0), q.stride(1), q.stride(2)
+    a.k_sb, a.k_ss, a.k_sh = k.stride(0), k.stride(1), k.stride(2)
+    a.v_sb, a.v_ss, a.v_sh = v.stride(0), v.stride(1), v.stride(2)
+    a.o_sb, a.o_ss, a.o_sh = out.stride(0), out.stride(1), out.stride(2)
+    a.B, a.H, a.Sq, a.Sk, a.D = B, H, Sq, Sk, D
+    a.softmax_scale = float(softmax_scale) if softmax_scale is not None else 0.0
+    qw = _f32("q_norm_weight", q_norm_weight, (D,))
+    kw = _f32("k_norm_weight", k_norm_weight, (D,))
+    a.q_norm_w, a.k_norm_w, a.norm_eps = _ptr(qw), _ptr(kw), float(norm_eps)
+    a.rope_mode = int(rope_mode)
+    if rope_mode != _lib.ROPE_NONE:
+        if rope_q is None:
+            raise ValueError("rope_mode set but rope_q tables missing")
+        if rope_k is None:
+            if Sq != Sk:
+                raise ValueError("rope_k tables are required when Sq != Sk")
+            rope_k = rope_q
+        qc, qs = _f32("rope_q cos", rope_q[0], (Sq, D // 2)), _f32("rope_q sin", rope_q[1], (Sq, D // 2))
+        kc, ks = _f32("rope_k cos", rope_k[0], (Sk, D // 2)), _f32("rope_k sin", rope_k[1], (Sk, D // 2))
+        a.q_rope_cos, a.q_rope_sin, a.k_rope_cos, a.k_rope_sin = qc.data_ptr(), qs.data_ptr(), kc.data_ptr(), ks.data_ptr()
+        keep += [qc, qs, kc, ks]
+    if key_mask is not None:
+        if tuple(key_mask.shape) != (B, Sk):
+            raise ValueError(f"key_mask must be [B, Sk] = {(B, Sk)}, got {tuple(key_mask.shape)}")
+        km = key_mask.to(torch.uint8).contiguous() if key_mask.dtype != torch.uint8 else key_mask.contiguous()
+        a.key_mask = km.data_ptr()
+        keep.append(km)
+    if block_mask is not None:
+        nrow = (Sq + 63) // 64
+        if block_mask.row_ptr.dtype != torch.int32 or block_mask.col_idx.dtype != torch.int32:
+            raise TypeError("block mask CSR arrays must be int32")
+        if block_mask.row_ptr.numel() != nrow + 1:
+            raise ValueError(f"block mask has {block_mask.row_ptr.numel() - 1} tile rows, need {nrow}")
+        a.blk_row_ptr, a.blk_col_idx = block_mask.row_ptr.data_ptr(), block_mask.col_idx.data_ptr()
+        keep += [block_mask.row_ptr, block_mask.col_idx]
+    a.flags = _lib.FLAG_FP8_QK if fp8_qk else 0
+    keep += [qw, kw]
+    return a, keep
+
+
+def workspace_bytes(args: _lib.AttnArgs) -> int:
+    n = _lib.load().pkh3_workspace_bytes(C.byref(args))
+    if n == 0:
+        raise _lib.Pkh3Error(_lib.PKH3_EARG, _lib.load().pkh3_last_error().decode())
+    return int(n)
+
+
+def attention(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+    workspace: Optional[torch.Tensor] = None, **opts,
+) -> torch.Tensor:
+    """softmax(norm_rope(q) norm_rope(k)^T * scale) v over ``[B, S, H, D]`` bf16 views (any strides
+    with a unit head-dim stride).  Keyword options are those of :func:`fill_args`.  Runs
+    asynchronously on the current stream and returns ``out`` ([B, Sq, H, D], bf16)."""
+    lib = _lib.load()
+    if out is None:
+        out = torch.empty((q.shape[0], q.shape[1], q.shape[2], q.shape[3]), dtype=torch.bfloat16, device=q.device)
+    args, keep = fill_args(q, k, v, out, **opts)
+    need = workspace_bytes(args)
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    args.workspace = workspace.data_ptr()
+    args.workspace_bytes = workspace.numel() * workspace.element_size()
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.pkh3_attn_fwd(C.byref(args), C.c_void_p(stream)))
+    # the workspace must outlive the kernels: tie it to the stream, not to this Python frame
+    workspace.record_stream(torch.cuda.current_stream())
+    return out
+
+
+def time_attention_kernel(q, k, v, *, iters: int = 10, **opts) -> float:
+    """Mean milliseconds per launch of the attention kernel alone (prologue excluded), measured with
+    HIP events inside the library on the current stream."""
+    lib = _lib.load()
+    out = torch.empty_like(q)
+    args, keep = fill_args(q, k, v, out, **opts)
+    ws = torch.empty(workspace_bytes(args), dtype=torch.uint8, device=q.device)
+    args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+    ms = C.c_float(0.0)
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.pkh3_attn_time_kernel(C.byref(args), C.c_void_p(stream), int(iters), C.byref(ms)))
+    return float(ms.value)
+
+
+def rope_tables(position_ids: torch.Tensor, axis_dims=(32, 48, 48), theta: float = 10000.0):
+    """cos/sin fp32 ``[S, 64]`` from the packed layout's ``position_ids`` ``[S, 3]`` float64 (device)."""
+    lib = _lib.load()
+    if position_ids.dim() != 2 or position_ids.shape[1] != 3:
+        raise ValueError(f"position_ids must be [S, 3], got {tuple(position_ids.shape)}")
+    if not position_ids.is_cuda:
+        raise ValueError("position_ids must live in device memory")
+    pos = position_ids.to(torch.float64).contiguous()
+    S = pos.shape[0]
+    cos = torch.empty((S, HEAD_DIM // 2), dtype=torch.float32, device=pos.device)
+    sin = torch.empty_like(cos)
+    dims = (C.c_int32 * 3)(*[int(x) for x in axis_dims])
+    with torch.cuda.device(pos.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.pkh3_rope_tables(pos.data_ptr(), S, dims, float(theta), cos.data_ptr(), sin.data_ptr(), C.c_void_p(stream)))
+    return cos, sin

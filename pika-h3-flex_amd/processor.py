@@ -1,0 +1,133 @@
+"""Attention processor for the H3 DiT blocks, in the shape diffusers' processor mechanism calls
+(``processor(attn, hidden_states, ...)``).
+
+The reference never builds attention itself: it loads ``diffusers.MiniMaxH3Transformer3DModel``
+(src/pika_h3/core/loader.py:11-18) whose attention modules own ``to_q / to_k / to_v / to_out.0``
+(the LoRA target list, src/pika_h3/core/loader.py:9) and calls the model with the packed-sequence
+tensors of src/pika_h3/core/wrapper.py:192-204 (``position_ids [S,3]`` float64 among them).  This
+processor is what gets attached to those modules: it runs the module's own projections (torch
+GEMMs, LoRA included), hands ``[B, S, H, D]`` strided views to libpkh3attn.so for
+QK-RMSNorm -> RoPE -> softmax(QK^T)V, and applies ``to_out``.
+
+Everything the pinned diffusers source alone could settle is an explicit constructor argument:
+RoPE pairing (``rope_mode``), axis split and theta, and where the norm weights are read from.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+from .ops import BlockMask, attention, rope_tables
+
+
+def _norm_weight(mod, dim: int, device) -> Optional[torch.Tensor]:
+    """fp32 weight of an RMSNorm-like module (``None`` module = no norm; no ``weight`` = ones)."""
+    if mod is None:
+        return None
+    w = getattr(mod, "weight", None)
+    if w is None:
+        return torch.ones(dim, dtype=torch.float32, device=device)
+    if w.numel() != dim:
+        raise ValueError(f"QK-norm weight has {w.numel()} elements; only per-head norm over D={dim} is supported")
+    return w.detach().to(device=device, dtype=torch.float32).contiguous()
+
+
+class PikaH3AttnProcessor:
+    """Drop-in attention processor backed by the gfx950 HIP kernels.
+
+    ``attn`` must expose ``to_q, to_k, to_v, to_out`` (``to_out[0]`` is the projection), ``heads``
+    and optionally ``norm_q / norm_k`` (RMSNorm over the head dim, ``eps`` attribute honoured).
+    """
+
+    def __init__(
+        self,
+        *,
+        rope_mode: int = _lib.ROPE_INTERLEAVED,
+        rope_axes_dims: Tuple[int, int, int] = (32, 48, 48),
+        rope_theta: float = 10000.0,
+        norm_eps: float = 1e-6,
+        fp8_qk: bool = False,
+    ):
+        self.rope_mode = int(rope_mode)
+        self.rope_axes_dims = tuple(int(x) for x in rope_axes_dims)
+        self.rope_theta = float(rope_theta)
+        self.norm_eps = float(norm_eps)
+        self.fp8_qk = bool(fp8_qk)
+        # position grids are constant across layers and denoising steps: one table per grid
+        self._rope_cache: Dict[Tuple[int, int, str], Tuple[torch.Tensor, torch.Tensor]] = {}
+        self._workspace: Optional[torch.Tensor] = None
+
+    def _tables(self, position_ids: torch.Tensor):
+        key = (position_ids.data_ptr(), position_ids.shape[0], str(position_ids.device))
+        hit = self._rope_cache.get(key)
+        if hit is None:
+            if len(self._rope_cache) >= 8:
+                self._rope_cache.pop(next(iter(self._rope_cache)))
+            hit = rope_tables(position_ids, self.rope_axes_dims, self.rope_theta)
+            self._rope_cache[key] = hit
+        return hit
+
+    def __call__(
+        self,
+        attn,
+        hidden_states: torch.Tensor,
+        encoder_hidden_states: Optional[torch.Tensor] = None,
+        attention_mask: Optional[torch.Tensor] = None,
+        *,
+        position_ids: Optional[torch.Tensor] = None,
+        rope_cos_sin: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+        block_mask: Optional[BlockMask] = None,
+        fp8_qk: Optional[bool] = None,
+    ) -> torch.Tensor:
+        """``hidden_states [B, S, H*D]`` -> ``[B, S, H*D]``.
+
+        Self-attention when ``encoder_hidden_states`` is None, else cross-attention with K/V from
+        ``encoder_hidden_states [B, Sk, C]`` and ``attention_mask`` a bool key-padding mask
+        ``[B, Sk]`` (True = attend).  RoPE applies to self-attention only, from ``position_ids
+        [S, 3]`` (or precomputed ``rope_cos_sin`` fp32 ``[S, D/2]`` tables).
+        """
+        if hidden_states.dim() != 3:
+            raise ValueError(f"hidden_states must be [B, S, C], got {tuple(hidden_states.shape)}")
+        B, S, _ = hidden_states.shape
+        H = int(attn.heads)
+        kv_src = hidden_states if encoder_hidden_states is None else encoder_hidden_states
+        q = attn.to_q(hidden_states)
+        k = attn.to_k(kv_src)
+        v = attn.to_v(kv_src)
+        D = q.shape[-1] // H
+        # [B, S, H*D] -> [B, S, H, D] views: no transpose copy, the kernels take the strides
+        q = q.view(B, S, H, D)
+        k = k.view(B, kv_src.shape[1], H, D)
+        v = v.view(B, kv_src.shape[1], H, D)
+        if q.dtype != torch.bfloat16:
+            q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
+
+        qn, kn = getattr(attn, "norm_q", None), getattr(attn, "norm_k", None)
+        eps = float(getattr(qn, "eps", None) or self.norm_eps)
+        opts = dict(
+            q_norm_weight=_norm_weight(qn, D, q.device),
+            k_norm_weight=_norm_weight(kn, D, q.device),
+            norm_eps=eps,
+            fp8_qk=self.fp8_qk if fp8_qk is None else bool(fp8_qk),
+            block_mask=block_mask,
+        )
+        if encoder_hidden_states is None:
+            if rope_cos_sin is None and position_ids is not None:
+                rope_cos_sin = self._tables(position_ids)
+            if rope_cos_sin is not None:
+                opts.update(rope_mode=self.rope_mode, rope_q=rope_cos_sin, rope_k=rope_cos_sin)
+            if attention_mask is not None:
+                opts.update(key_mask=attention_mask)
+        else:
+            if attention_mask is not None:
+                opts.update(key_mask=attention_mask)
+
+        need_ws = self._workspace
+        out = attention(q, k, v, workspace=need_ws, **opts)
+        out = out.view(B, S, H * D).to(hidden_states.dtype)
+        out = attn.to_out[0](out)
+        if len(attn.to_out) > 1:
+            out = attn.to_out[1](out)
+        return out

@@ -1,0 +1,153 @@
+"""GPU parity: the HIP path, called through the C ABI, against the float64 oracle on the same
+seeded inputs.  Tolerance for the bf16 paths (from the benchmark contract): max-abs <= 2e-2 and
+cosine >= 0.9999 versus the float64/fp32 reference."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS = 2e-2
+MIN_COS = 0.9999
+
+
+def _oracle():
+    from oracle import attention_oracle as O
+
+    return O
+
+
+def _rand(shape, gen, std=1.0):
+    return (torch.randn(shape, generator=gen, dtype=torch.float32) * std).to(torch.bfloat16)
+
+
+def _run_and_check(B, Sq, Sk, H, *, seed=0, norm=True, rope_mode=0, mask=None, std=1.0, min_cos=MIN_COS,
+                   max_abs=MAX_ABS, weight_random=False):
+    import pika_h3_flex_amd as pk
+
+    O = _oracle()
+    D = 128
+    gen = torch.Generator().manual_seed(seed)
+    q, k, v = _rand((B, Sq, H, D), gen, std), _rand((B, Sk, H, D), gen, std), _rand((B, Sk, H, D), gen)
+    qw = kw = None
+    if norm:
+        if weight_random:
+            qw = 1.0 + 0.2 * torch.randn(D, generator=gen)
+            kw = 1.0 + 0.2 * torch.randn(D, generator=gen)
+        else:
+            qw, kw = torch.ones(D), torch.ones(D)
+    rope_q = rope_k = None
+    if rope_mode:
+        posq = torch.rand((Sq, 3), generator=gen, dtype=torch.float64) * torch.tensor([30.0, 29.0, 51.0], dtype=torch.float64)
+        posk = posq if Sq == Sk else torch.rand((Sk, 3), generator=gen, dtype=torch.float64) * 40.0
+        rope_q = O.rope_tables(posq)
+        rope_k = O.rope_tables(posk)
+    ref = O.reference_layer(q, k, v, q_norm_weight=qw, k_norm_weight=kw, rope_q=rope_q, rope_k=rope_k,
+                            rope_mode=rope_mode, key_mask=mask)
+    dev = "cuda"
+    f32 = lambda t: None if t is None else t.to(torch.float32).contiguous().to(dev)
+    opts = dict(q_norm_weight=f32(qw), k_norm_weight=f32(kw), norm_eps=1e-6, rope_mode=rope_mode)
+    if rope_mode:
+        opts.update(rope_q=(f32(rope_q[0]), f32(rope_q[1])), rope_k=(f32(rope_k[0]), f32(rope_k[1])))
+    if mask is not None:
+        opts.update(key_mask=mask.to(dev))
+    out = pk.attention(q.to(dev), k.to(dev), v.to(dev), **opts)
+    torch.cuda.synchronize()
+    out = out.cpu()
+    assert torch.isfinite(out.float()).all()
+    err, cos = O.max_abs_and_cosine(out, ref)
+    print(f"B={B} Sq={Sq} Sk={Sk} H={H} rope={rope_mode} mask={mask is not None}: max_abs={err:.3e} cos={cos:.7f}", flush=True)
+    assert err <= max_abs and cos >= min_cos
+    return out, ref
+
+
+def test_plumbing_config():
+    """B=1, H=4, S=1024, D=128, N(0,1) inputs, QK-RMSNorm (eps 1e-6, unit weight), no mask."""
+    _run_and_check(1, 1024, 1024, 4, seed=1)
+
+
+@pytest.mark.parametrize("S", [1, 7, 64, 65, 200, 257, 1000])
+def test_ragged_lengths(S):
+    _run_and_check(1, S, S, 2, seed=S)
+
+
+@pytest.mark.parametrize("Sq,Sk", [(5, 300), (300, 5), (513, 129), (64, 4096)])
+def test_rectangular(Sq, Sk):
+    _run_and_check(1, Sq, Sk, 3, seed=Sq + Sk)
+
+
+def test_batch_and_heads():
+    _run_and_check(3, 130, 130, 5, seed=9)
+
+
+@pytest.mark.parametrize("mode", [1, 2])
+def test_rope_modes(mode):
+    _run_and_check(1, 333, 333, 2, seed=40 + mode, rope_mode=mode, weight_random=True)
+
+
+def test_no_norm_small_logits():
+    _run_and_check(1, 256, 256, 2, seed=5, norm=False, std=0.3)
+
+
+def test_key_mask_suffix_and_scattered():
+    gen = torch.Generator().manual_seed(77)
+    B, Sk = 2, 512
+    mask = torch.zeros((B, Sk), dtype=torch.bool)
+    mask[0, :137] = True                              # suffix padding
+    mask[1] = torch.rand(Sk, generator=gen) < 0.4     # scattered
+    _run_and_check(B, 200, Sk, 2, seed=6, mask=mask)
+
+
+def test_key_mask_all_valid_equals_no_mask():
+    import pika_h3_flex_amd as pk
+
+    gen = torch.Generator().manual_seed(3)
+    q, k, v = (_rand((1, 100, 2, 128), gen).cuda() for _ in range(3))
+    a = pk.attention(q, k, v)
+    b = pk.attention(q, k, v, key_mask=torch.ones((1, 100), dtype=torch.bool, device="cuda"))
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_fully_masked_rows_are_zero():
+    import pika_h3_flex_amd as pk
+
+    gen = torch.Generator().manual_seed(4)
+    q, k, v = (_rand((1, 70, 2, 128), gen).cuda() for _ in range(3))
+    out = pk.attention(q, k, v, key_mask=torch.zeros((1, 70), dtype=torch.bool, device="cuda"))
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(out) == 0
+
+
+def test_strided_views_no_copy():
+    """q/k/v as column slices of one fused [B, S, 3*H*D] projection output."""
+    import pika_h3_flex_amd as pk
+
+    O = _oracle()
+    gen = torch.Generator().manual_seed(12)
+    B, S, H, D = 1, 150, 3, 128
+    qkv = _rand((B, S, 3 * H * D), gen)
+    q, k, v = (qkv[..., i * H * D:(i + 1) * H * D].view(B, S, H, D) for i in range(3))
+    ref = O.reference_layer(q, k, v)
+    g = qkv.cuda()
+    qg, kg, vg = (g[..., i * H * D:(i + 1) * H * D].view(B, S, H, D) for i in range(3))
+    assert not qg.is_contiguous()
+    out = pk.attention(qg, kg, vg)
+    torch.cuda.synchronize()
+    err, cos = O.max_abs_and_cosine(out.cpu(), ref)
+    assert err <= MAX_ABS and cos >= MIN_COS
+
+
+def test_rope_tables_kernel():
+    import pika_h3_flex_amd as pk
+
+    O = _oracle()
+    from pika_h3_flex_amd.layout import audio_position_ids, video_position_ids
+
+    pos = torch.cat([video_position_ids(5, 6, 7), audio_position_ids(40)], 0)
+    cos, sin = pk.rope_tables(pos.cuda())
+    rc, rs = O.rope_tables(pos)
+    torch.cuda.synchronize()
+    assert (cos.cpu().double() - rc).abs().max() < 1e-6
+    assert (sin.cpu().double() - rs).abs().max() < 1e-6
