@@ -12,6 +12,8 @@
 //   O^T += V^T P^T     A = V image (LDS), B = P packed to bf16 straight from the S^T registers
 // The transposed formulation keeps every per-query quantity (max, sum, rescale factor) a per-lane
 // scalar: no cross-lane traffic in the rescale, none between the two GEMMs.
+#include <stdlib.h>
+
 #include "pkh3_common.h"
 #include "pkh3_internal.h"
 
@@ -38,6 +40,128 @@ __device__ __forceinline__ void prefetch_tile(const char* tile, char* buf, int w
   }
 }
 
+// Per-wave register state.
+struct WaveState {
+  bf16x8 qf[2][8];      // Q images: [query block][k-step]
+  f32x16 sa[2], sb[2];  // S^T of two consecutive 32-key sub-tiles (ping-pong), per query block
+  bf16x8 pa[2][2], pb[2][2];  // P of two consecutive sub-tiles: [query block][k-step of 16 keys]
+  f32x16 o[2][4];       // O^T accumulators: [query block][32-wide block of d]
+  float m[2], l[2];     // running row max (scaled, log2 domain) and per-half-wave row sum
+  float alpha[2];       // factor the last step lowered the old terms by (1 unless the max moved)
+};
+
+constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
+
+__device__ __forceinline__ float max_across_halves(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// One pipeline step on 32-key sub-tiles, three independent instruction streams the scheduler may interleave:
+//   MFMA:  S_next = K'(u+1) Q'^T        (16 MFMAs, K images from LDS at kptr)
+//   MFMA:  O^T   += V(u-1)^T P_prev     (16 MFMAs, V images from LDS at vptr)           [DO_PV]
+//   VALU:  P_cur = softmax numerators of S_cur (sub-tile u), running max / sum update
+// `lim`: number of keys of sub-tile u that exist (only read when MASK).
+template <bool DO_PV, bool MASK>
+__device__ __forceinline__ void pipe_step(const char* kptr, const char* vptr, const bf16x8 (&qf)[2][8],
+                                          const f32x16 (&s_cur)[2], f32x16 (&s_nxt)[2], const bf16x8 (&p_prev)[2][2],
+                                          bf16x8 (&p_cur)[2][2], f32x16 (&o)[2][4], float (&m)[2], float (&l)[2],
+                                          float (&alpha)[2], float c, int lim, int lane) {
+  const int hh = lane >> 5;
+  // ---- rescale O^T where the previous step moved the running max: after that step's P.V (sub-tile
+  //      u-2), before this step's P.V (sub-tile u-1, whose numerators use the new max).  Rare.
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    if (__any(alpha[qb] != 1.0f)) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha[qb];
+    }
+  }
+  // ---- QK^T of the next sub-tile
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    const bf16x8 kf = *(const bf16x8*)(kptr + (ks * 64 + lane) * 16);
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      if (ks == 0) {
+        f32x16 z;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) z[i] = 0.f;
+        s_nxt[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], z, 0, 0, 0);
+      } else {
+        s_nxt[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], s_nxt[qb], 0, 0, 0);
+      }
+    }
+  }
+  // ---- P.V of the previous sub-tile
+  if constexpr (DO_PV) {
+#pragma unroll
+    for (int b2 = 0; b2 < 2; ++b2)
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        const bf16x8 vf = *(const bf16x8*)(vptr + ((b2 * 4 + db) * 64 + lane) * 16);
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+          o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_prev[qb][b2], o[qb][db], 0, 0, 0);
+      }
+  }
+  // ---- softmax numerators of the current sub-tile
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    f32x16 s = s_cur[qb];
+    if constexpr (MASK) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = 8 * (i / 4) + 4 * hh + (i % 4);
+        if (key >= lim) s[i] = -INFINITY;
+      }
+    }
+    float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+    for (int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
+    mx = fmaxf(mx, s[15]);
+    mx = max_across_halves(mx) * c;
+    // raise the running max only when it is exceeded by more than the slack: P stays <= 2^slack and
+    // the O^T rescale below becomes rare
+    const float m_old = m[qb];
+    const float m_new = (mx > m_old + kRescaleSlack) ? mx : m_old;
+    alpha[qb] = __builtin_amdgcn_exp2f(m_old - m_new);
+    m[qb] = m_new;
+    float rsum = 0.f;
+#pragma unroll
+    for (int b2 = 0; b2 < 2; ++b2) {
+      bf16x8 pk;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pk[j] = (__bf16)__builtin_amdgcn_exp2f(fmaf(s[8 * b2 + j], c, -m_new));
+      // row sum over the bf16-rounded values, the same numbers the P.V MFMA consumes
+      const bf16x2 one2 = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+      for (int j = 0; j < 8; j += 2) {
+        const bf16x2 pr = {pk[j], pk[j + 1]};
+        rsum = __builtin_amdgcn_fdot2_f32_bf16(pr, one2, rsum, false);
+      }
+      p_cur[qb][b2] = pk;
+    }
+    l[qb] = l[qb] * alpha[qb] + rsum;
+  }
+  // keep the numerators' computation inside this step (next to the MFMAs it overlaps with)
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int b2 = 0; b2 < 2; ++b2) asm volatile("" : "+v"(p_cur[qb][b2]));
+  // register-file hints: the S^T results feed VALU work (VGPRs), O^T is only touched by MFMAs (AGPRs)
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) asm volatile("" : "+v"(s_nxt[qb]));
+#ifdef PKH3_HINT_O_AGPR
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int db = 0; db < 4; ++db) asm volatile("" : "+a"(o[qb][db]));
+#endif
+}
+
 __global__ __launch_bounds__(256, 1) void attn_fwd_dense_kernel(FwdParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[kNBuf][kKvTileBytes];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -52,124 +176,110 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_dense_kernel(FwdParams p) {
   if (lin >= total) return;
   const int bh = lin / nQt, qt = lin % nQt;
   const int b = bh / p.H, h = bh % p.H;
+  const int q64 = qt * kWaves + wave;
 
   const int sk = p.row_cnt ? p.row_cnt[b] : p.Sk;
   const int nt = (sk + kTileKeys - 1) / kTileKeys;
   const char* kv = p.kv + (int64_t)bh * p.kv_bh_stride;
 
-  if (nt > 0) prefetch_tile(kv, lds[0], wave, lane);
-
-  // Q images for this wave's 64 queries
-  const int q64 = qt * kWaves + wave;
-  bf16x8 qf[2][8];
-  {
-    const bf16x8* qsrc = (const bf16x8*)(p.qp + (int64_t)bh * p.q_bh_stride + (int64_t)q64 * p.q_blk_stride);
+  WaveState w;
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) qf[qb][ks] = qsrc[(qb * 8 + ks) * 64 + lane];
-  }
-
-  f32x16 o[2][4];
-#pragma unroll
-  for (int qb = 0; qb < 2; ++qb)
+  for (int qb = 0; qb < 2; ++qb) {
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
-  float m[2] = {-INFINITY, -INFINITY};
-  float l[2] = {0.f, 0.f};
-  const float c = p.c;
+      for (int i = 0; i < 16; ++i) w.o[qb][db][i] = 0.f;
+    w.m[qb] = -INFINITY;
+    w.l[qb] = 0.f;
+    w.alpha[qb] = 1.0f;
+  }
 
-  for (int t = 0; t < nt; ++t) {
-    // tile t has landed (this wave's part: vmcnt; everyone's: barrier); the barrier also says every
-    // wave is done reading the buffer tile t+1 goes into (it held tile t-2).
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (t + 1 < nt) prefetch_tile(kv + (int64_t)(t + 1) * p.kv_tile_stride, lds[(t + 1) % kNBuf], wave, lane);
-    const char* kbuf = lds[t % kNBuf];
-    const char* vbuf = kbuf + kKTileBytes;
-
-    f32x16 s[2][2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+  if (nt > 0) {
+    prefetch_tile(kv, lds[0], wave, lane);
+    {
+      const bf16x8* qsrc = (const bf16x8*)(p.qp + (int64_t)bh * p.q_bh_stride + (int64_t)q64 * p.q_blk_stride);
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[qb][kb][i] = 0.f;
+        for (int ks = 0; ks < 8; ++ks) w.qf[qb][ks] = qsrc[(qb * 8 + ks) * 64 + lane];
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (nt > 1) prefetch_tile(kv + (int64_t)p.kv_tile_stride, lds[1], wave, lane);
+
+    // pre-step: S_a = QK^T of sub-tile (0, 0)
+    {
+      const char* kptr = lds[0];
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) w.sa[qb][i] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
-        const bf16x8 kf = *(const bf16x8*)(kbuf + ((kb * 8 + ks) * 64 + lane) * 16);
+        const bf16x8 kf = *(const bf16x8*)(kptr + (ks * 64 + lane) * 16);
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb)
-          s[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], s[qb][kb], 0, 0, 0);
+          w.sa[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, w.qf[qb][ks], w.sa[qb], 0, 0, 0);
       }
     }
 
-    if (t == nt - 1 && (sk & (kTileKeys - 1))) {
-      const int lim = sk - t * kTileKeys;  // keys of this tile that exist
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = kb * 32 + 8 * (i / 4) + 4 * hh + (i % 4);
-          if (key >= lim) {
-            s[0][kb][i] = -INFINITY;
-            s[1][kb][i] = -INFINITY;
-          }
-        }
+    const float c = p.c;
+    const int last_lim = sk - (nt - 1) * kTileKeys;  // keys that exist in the last tile (1..64)
+    // Ring slots of tiles t-1, t, t+1.  Each iteration runs the two sub-tile steps of tile t:
+    //   step (t,0): S_b = QK^T(t,1);   O += P_b V(t-1,1);  P_a = softmax(S_a)
+    //   sync:       tile t+1 has landed (own part: vmcnt, everyone's: barrier); all waves are past
+    //               V(t-1), so its slot takes tile t+2
+    //   step (t,1): S_a = QK^T(t+1,0); O += P_a V(t,0);    P_b = softmax(S_b)
+    // The first tile has no previous P.V and the last one masks the keys past the end; both are
+    // peeled so that the steady-state loop body has no branches besides the rare O^T rescale.
+    int buf_p = kNBuf - 1, buf = 0, buf_n = 1;
+#define PKH3_TILE_ITER(T, DO_PV0, MASKED)                                                                         \
+  {                                                                                                               \
+    pipe_step<DO_PV0, MASKED>(lds[buf] + 8 * 1024, lds[buf_p] + kKTileBytes + 8 * 1024, w.qf, w.sa, w.sb, w.pb,   \
+                              w.pa, w.o, w.m, w.l, w.alpha, c, last_lim, lane);                                            \
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                              \
+    __syncthreads();                                                                                              \
+    if ((T) + 2 < nt) prefetch_tile(kv + (int64_t)((T) + 2) * p.kv_tile_stride, lds[buf_p], wave, lane);          \
+    pipe_step<true, MASKED>(lds[buf_n], lds[buf] + kKTileBytes, w.qf, w.sb, w.sa, w.pa, w.pb, w.o, w.m, w.l,      \
+                            w.alpha, c, last_lim - 32, lane);                                                                 \
+    buf_p = buf;                                                                                                  \
+    buf = buf_n;                                                                                                  \
+    buf_n = buf_n + 1 == kNBuf ? 0 : buf_n + 1;                                                                   \
+  }
+    if (nt == 1) {
+      PKH3_TILE_ITER(0, false, true)
+    } else {
+      PKH3_TILE_ITER(0, false, false)
+      for (int t = 1; t < nt - 1; ++t) PKH3_TILE_ITER(t, true, false)
+      PKH3_TILE_ITER(nt - 1, true, true)
     }
-
-    bf16x8 pf[2][2][2];
+#undef PKH3_TILE_ITER
+    // drain: O += P_b V(nt-1, 1)
+    {
+      const char* vptr = lds[buf_p] + kKTileBytes + 8 * 1024;
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      float mx = s[qb][0][0];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[qb][kb][i]);
-      mx = fmaxf(mx, xhalf(mx));
-      const float m_new = fmaxf(m[qb], mx * c);
-      const float alpha = __builtin_amdgcn_exp2f(m[qb] - m_new);
-      m[qb] = m_new;
-      float rsum = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int b2 = 0; b2 < 2; ++b2)
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const float e = __builtin_amdgcn_exp2f(fmaf(s[qb][kb][8 * b2 + j], c, -m_new));
-            rsum += e;
-            pf[qb][kb][b2][j] = (__bf16)e;
-          }
-      l[qb] = l[qb] * alpha + rsum;
-      if (__any(alpha != 1.0f)) {
+      for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
-      }
-    }
-
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+          for (int i = 0; i < 16; ++i) w.o[qb][db][i] *= w.alpha[qb];
 #pragma unroll
       for (int b2 = 0; b2 < 2; ++b2)
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
-          const bf16x8 vf = *(const bf16x8*)(vbuf + (((kb * 2 + b2) * 4 + db) * 64 + lane) * 16);
+          const bf16x8 vf = *(const bf16x8*)(vptr + ((b2 * 4 + db) * 64 + lane) * 16);
 #pragma unroll
           for (int qb = 0; qb < 2; ++qb)
-            o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[qb][kb][b2], o[qb][db], 0, 0, 0);
+            w.o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, w.pb[qb][b2], w.o[qb][db], 0, 0, 0);
         }
+    }
   }
 
   // epilogue: O = O^T / l, bf16, 8-byte stores (4 consecutive d per register group)
   __bf16* ob = (__bf16*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {
-    const float lt = l[qb] + xhalf(l[qb]);
+    const float lt = w.l[qb] + xhalf(w.l[qb]);
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     const int q = q64 * 64 + qb * 32 + (lane & 31);
     if (q < p.Sq) {
@@ -178,12 +288,143 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_dense_kernel(FwdParams p) {
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          bf16x4 w;
+          bf16x4 wv;
 #pragma unroll
-          for (int rr = 0; rr < 4; ++rr) w[rr] = (__bf16)(o[qb][db][4 * g + rr] * inv);
-          *(bf16x4*)(orow + 32 * db + 8 * g + 4 * hh) = w;
+          for (int rr = 0; rr < 4; ++rr) wv[rr] = (__bf16)(w.o[qb][db][4 * g + rr] * inv);
+          *(bf16x4*)(orow + 32 * db + 8 * g + 4 * hh) = wv;
         }
     }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Variant: 8 waves (two per SIMD), 32 queries per wave.  The two waves sharing a SIMD drift out of
+// phase, so one wave's softmax VALU work overlaps the other's MFMAs without software pipelining.
+__global__ __launch_bounds__(512, 1) void attn_fwd_w8_kernel(FwdParams p) {
+  __shared__ __attribute__((aligned(1024))) char lds[kNBuf][kKvTileBytes];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int hh = lane >> 5;
+  const int nQt = p.nQ64 / kWaves;
+  const int total = p.B * p.H * nQt;
+  const int per_xcd = (total + 7) / 8;
+  const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (lin >= total) return;
+  const int bh = lin / nQt, qt = lin % nQt;
+  const int b = bh / p.H, h = bh % p.H;
+  const int q32 = qt * 8 + wave;  // 32-query block of this wave
+
+  const int sk = p.row_cnt ? p.row_cnt[b] : p.Sk;
+  const int nt = (sk + kTileKeys - 1) / kTileKeys;
+  const char* kv = p.kv + (int64_t)bh * p.kv_bh_stride;
+
+  auto prefetch8 = [&](const char* tile, char* buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int chunk = wave * 4 + i;
+      lds_dma16(tile + chunk * 1024 + lane * 16, buf + chunk * 1024);
+    }
+  };
+  if (nt > 0) prefetch8(kv, lds[0]);
+
+  bf16x8 qf[8];
+  {
+    const bf16x8* qsrc = (const bf16x8*)(p.qp + (int64_t)bh * p.q_bh_stride + (int64_t)(q32 >> 1) * p.q_blk_stride) + (q32 & 1) * 8 * 64;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = qsrc[ks * 64 + lane];
+  }
+  f32x16 o[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  const float c = p.c;
+
+  for (int t = 0; t < nt; ++t) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (t + 1 < nt) prefetch8(kv + (int64_t)(t + 1) * p.kv_tile_stride, lds[(t + 1) % kNBuf]);
+    const char* kbuf = lds[t % kNBuf];
+    const char* vbuf = kbuf + kKTileBytes;
+
+    f32x16 s[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 kf = *(const bf16x8*)(kbuf + ((kb * 8 + ks) * 64 + lane) * 16);
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[kb], 0, 0, 0);
+      }
+    }
+    if (t == nt - 1 && (sk & (kTileKeys - 1))) {
+      const int lim = sk - t * kTileKeys;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = kb * 32 + 8 * (i / 4) + 4 * hh + (i % 4);
+          if (key >= lim) s[kb][i] = -INFINITY;
+        }
+    }
+    float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(fmaxf(mx, s[0][i]), s[1][i]);
+    mx = max_across_halves(mx) * c;
+    const float m_new = (mx > m + kRescaleSlack) ? mx : m;
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+    m = m_new;
+    bf16x8 pf[2][2];
+    float rsum = 0.f;
+    const bf16x2 one2 = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int b2 = 0; b2 < 2; ++b2) {
+        bf16x8 pk;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pk[j] = (__bf16)__builtin_amdgcn_exp2f(fmaf(s[kb][8 * b2 + j], c, -m_new));
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+          const bf16x2 pr = {pk[j], pk[j + 1]};
+          rsum = __builtin_amdgcn_fdot2_f32_bf16(pr, one2, rsum, false);
+        }
+        pf[kb][b2] = pk;
+      }
+    l = l * alpha + rsum;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    }
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int b2 = 0; b2 < 2; ++b2)
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const bf16x8 vf = *(const bf16x8*)(vbuf + (((kb * 2 + b2) * 4 + db) * 64 + lane) * 16);
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kb][b2], o[db], 0, 0, 0);
+        }
+  }
+
+  __bf16* ob = (__bf16*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
+  const float lt = l + xhalf(l);
+  const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+  const int q = q32 * 32 + (lane & 31);
+  if (q < p.Sq) {
+    __bf16* orow = ob + (int64_t)q * p.o_ss;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        bf16x4 wv;
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) wv[rr] = (__bf16)(o[db][4 * g + rr] * inv);
+        *(bf16x4*)(orow + 32 * db + 8 * g + 4 * hh) = wv;
+      }
   }
 }
 
@@ -191,7 +432,11 @@ hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
   const int nQt = p.nQ64 / kWaves;
   const int total = p.B * p.H * nQt;
   const int per_xcd = (total + 7) / 8;
-  hipLaunchKernelGGL(attn_fwd_dense_kernel, dim3(per_xcd * 8), dim3(256), 0, st, p);
+  static const int variant = getenv("PKH3_KERNEL") ? atoi(getenv("PKH3_KERNEL")) : 0;
+  if (variant == 1)
+    hipLaunchKernelGGL(attn_fwd_w8_kernel, dim3(per_xcd * 8), dim3(512), 0, st, p);
+  else
+    hipLaunchKernelGGL(attn_fwd_dense_kernel, dim3(per_xcd * 8), dim3(256), 0, st, p);
   return hipGetLastError();
 }
 
