@@ -53,6 +53,8 @@ int validate(const pkh3_attn_args* a, bool pointers) {
   if ((a->blk_row_ptr == nullptr) != (a->blk_col_idx == nullptr))
     return fail(PKH3_ENULL, "blk_row_ptr and blk_col_idx must be given together");
   if (a->blk_row_ptr && a->key_mask) return fail(PKH3_EUNSUPPORTED, "block-sparse map together with a key mask is not supported");
+  if ((a->flags & PKH3_FLAG_FP8_QK) && a->key_mask)
+    return fail(PKH3_EUNSUPPORTED, "fp8 QK^T together with a key mask is not supported");
   if (!pointers) return PKH3_OK;
   int rc;
   if ((rc = check_tensor("q", a->q, a->q_sb, a->q_ss, a->q_sh, a->B, a->H))) return rc;
@@ -87,6 +89,8 @@ WsPlan plan(const pkh3_attn_args* a) {
   w.kscale_off = off; if (fp8) off = align_up(off + bh * w.nKt * sizeof(float), 256);
   w.cnt_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * sizeof(int), 256);
   w.idx_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * a->Sk * sizeof(int), 256);
+  w.plan_off = off;   if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / 4) * w.nKt * sizeof(int), 256);
+  w.plan_cnt_off = off; if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / 4) * sizeof(int), 256);
   w.total = off;
   return w;
 }
@@ -143,7 +147,9 @@ void build(const pkh3_attn_args* a, Launch& L) {
   f.B = a->B; f.H = a->H; f.Sq = a->Sq; f.Sk = a->Sk; f.nQ64 = L.w.nQ64; f.nKt = L.w.nKt;
   const float scale = a->softmax_scale > 0.f ? a->softmax_scale : 1.0f / sqrtf((float)kD);
   f.c = scale * kLog2e;
-  f.blk_row_ptr = a->blk_row_ptr; f.blk_col_idx = a->blk_col_idx;
+  f.plan = a->blk_row_ptr ? (const int*)(ws + L.w.plan_off) : nullptr;
+  f.plan_cnt = a->blk_row_ptr ? (const int*)(ws + L.w.plan_cnt_off) : nullptr;
+  f.plan_stride = L.w.nKt;
   f.qscale = q.scale_out; f.kscale = k.scale_out; f.fp8 = fp8;
 }
 
@@ -155,6 +161,12 @@ int run_prologue(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
   hipError_t e;
   if (a->key_mask) {
     if ((e = launch_mask_compact(a->key_mask, a->B, a->Sk, L.idx, L.cnt, st)) != hipSuccess) return hip_fail(e, "mask_compact");
+  }
+  if (a->blk_row_ptr) {
+    char* ws = (char*)a->workspace;
+    if ((e = launch_sparse_plan(a->blk_row_ptr, a->blk_col_idx, (a->Sq + 63) / 64, L.w.nQ64, L.w.nKt, (int*)(ws + L.w.plan_off),
+                                L.w.nKt, (int*)(ws + L.w.plan_cnt_off), st)) != hipSuccess)
+      return hip_fail(e, "sparse plan");
   }
   if ((e = launch_qk_prologue(L.qp, st)) != hipSuccess) return hip_fail(e, "q prologue");
   if ((e = launch_qk_prologue(L.kp, st)) != hipSuccess) return hip_fail(e, "k prologue");

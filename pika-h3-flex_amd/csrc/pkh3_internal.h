@@ -12,7 +12,7 @@ struct WsPlan {
   int nKt;       // 64-key tiles
   int kvTileBytes;  // bytes of one [K tile | V tile] record
   int qBlkBytes;    // bytes of one 64-query block of Q images
-  size_t q_off, kv_off, qscale_off, kscale_off, cnt_off, idx_off, total;
+  size_t q_off, kv_off, qscale_off, kscale_off, cnt_off, idx_off, plan_off, plan_cnt_off, total;
 };
 
 // One side (Q or K) of the normalise + rotate + lay-out pass.
@@ -59,8 +59,9 @@ struct FwdParams {
   int B, H, Sq, Sk;
   int nQ64, nKt;
   float c;                  // softmax_scale * log2(e)
-  const int* blk_row_ptr;
-  const int* blk_col_idx;
+  const int* plan;          // block-sparse: per query tile (256 queries) the union tile list, or null
+  const int* plan_cnt;      // [nQ64/4] entries per query tile
+  int plan_stride;          // ints between consecutive query tiles' lists
   const float* qscale;      // [B*H, nQ64]
   const float* kscale;      // [B*H, nKt]
   int fp8;
@@ -70,6 +71,8 @@ hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int
 hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st);
 hipError_t launch_v_prologue(const VPrologueParams& p, hipStream_t st);
 hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st);
+hipError_t launch_sparse_plan(const int* row_ptr, const int* col_idx, int nRow64, int nQ64, int nKt, int* plan,
+                              int plan_stride, int* plan_cnt, hipStream_t st);
 hipError_t launch_rope_tables(const double* pos, int S, const int* axis_dims, double theta, float* cos_out,
                               float* sin_out, hipStream_t st);
 
