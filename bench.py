@@ -1,0 +1,133 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+Workload (default): the 480p video self-attention layer -- B=1, H=24, D=128, S = 31 x (30 x 52) =
+48,360 tokens; hidden states ~ N(0,1) projected by random-init Wq/Wk/Wv (std 0.02), QK-RMSNorm
+(eps 1e-6, unit weight), 3-axis RoPE (32/48/48, theta 1e4); non-causal, no mask.  A "step" is one
+layer call through the C ABI: prologue kernels (norm + RoPE + operand layout of Q, K, V) plus the
+attention kernel, inputs resident in HBM.
+
+Prints ONE JSON line: `value` = 4*Sq*Sk*D*H / step time in TFLOP/s; `roofline` prices the attention
+kernel alone (HIP events on its stream, inside the library) against the bf16 dense MFMA peak;
+`cpu_baseline` times torch's CPU scaled_dot_product_attention path on a declared query-row sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}  # MI355X dense MFMA, published
+HBM_PEAK_GBS = 8000.0
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="480p", choices=["plumbing", "480p", "768p", "joint", "cross", "480p-sparse", "480p-sparse-fp8", "480p-fp8"])
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--cpu-rows", type=int, default=16384, help="query rows of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--kernel-iters", type=int, default=10)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU over the full local sequence (no sequence-parallel split, "
+              "no collectives); --gpus must be 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import pika_h3_flex_amd as pk
+    from pika_h3_flex_amd import workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP library is the only compute path", file=sys.stderr)
+        return 2
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+
+    base = args.workload.split("-")[0]
+    inp = workloads.make(base, seed=args.seed, device=dev)
+    B, Sq, H, D = inp.q.shape
+    Sk = inp.k.shape[1]
+    ones = torch.ones(D, dtype=torch.float32, device=dev)
+    opts = dict(q_norm_weight=ones, k_norm_weight=ones, norm_eps=1e-6)
+    tabs = None
+    if inp.position_ids is not None:
+        tabs = pk.rope_tables(inp.position_ids)
+        opts.update(rope_mode=pk.ROPE_INTERLEAVED, rope_q=tabs)
+    if inp.key_mask is not None:
+        opts.update(key_mask=inp.key_mask)
+    density = 1.0
+    fp8 = args.workload.endswith("fp8")
+    if "sparse" in args.workload:
+        tm = pk.local_window_tile_map(Sq, inp.tokens_per_frame, window_frames=2, global_fraction=0.10, seed=args.seed)
+        density = float(tm.float().mean())
+        opts.update(block_mask=pk.BlockMask.from_dense(tm, device=dev))
+    if fp8:
+        opts.update(fp8_qk=True)
+    flops = inp.flops * density
+
+    out = torch.empty_like(inp.q)
+    args_ws, _keep = pk.ops.fill_args(inp.q, inp.k, inp.v, out, **opts)
+    ws = torch.empty(pk.ops.workspace_bytes(args_ws), dtype=torch.uint8, device=dev)
+
+    def step():
+        pk.attention(inp.q, inp.k, inp.v, out=out, workspace=ws, **opts)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = flops / (ms_per_step * 1e-3) / 1e12
+
+    kernel_ms = pk.time_attention_kernel(inp.q, inp.k, inp.v, iters=args.kernel_iters, **opts)
+    achieved = flops / (kernel_ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS["fp8" if fp8 else "bf16"]
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4), "traffic": None, "kernel": "attn_fwd_kernel",
+                "kernel_ms": round(kernel_ms, 4), "flops_per_launch": flops}
+
+    cpu = None
+    if args.cpu_rows > 0:
+        from oracle import cpu_sdpa
+
+        rows = min(args.cpu_rows, Sq)
+        cpu_opts = dict(q_norm_weight=ones, k_norm_weight=ones, eps=1e-6, dtype=torch.float32)
+        if tabs is not None:
+            cpu_opts.update(rope_q=tabs)
+        if inp.key_mask is not None:
+            cpu_opts.update(key_mask=inp.key_mask.cpu())
+        secs, threads = cpu_sdpa.time_cpu_baseline(inp.q, inp.k, inp.v, sample_rows=rows, **cpu_opts)
+        sk_eff = Sk if inp.key_mask is None else int(inp.key_mask.sum())
+        cpu_flops = 4.0 * rows * sk_eff * D * H
+        cpu = {"value": round(cpu_flops / secs / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+               "sample": f"torch CPU F.scaled_dot_product_attention fp32 (+RMSNorm, RoPE in torch) on the first {rows} of {Sq} "
+                         f"query rows x all {Sk} keys x {H} heads, dense, one call of {secs:.2f} s; rate scales linearly in rows"}
+
+    line = {
+        "metric": "attention TFLOP/s (4*Sq*Sk*D*H per layer call; prologue + attention kernel)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8-e4m3 QK^T + bf16 PV" if fp8 else "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.workload} attention layer: B={B}, H={H}, D={D}, Sq={Sq}, Sk={Sk}, "
+                               f"QK-RMSNorm + 3-axis RoPE, non-causal" + (f", block-sparse density {density:.3f}" if density < 1 else ""),
+                   "seed": args.seed, "pct_of_mfma_peak": round(100.0 * value / peak, 2)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

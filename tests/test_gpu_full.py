@@ -1,0 +1,226 @@
+"""GPU parity at the benchmark's full sizes and against the committed golden vectors.
+
+Full-size checks combine (a) the float64 oracle on sampled query rows x a few heads over the full
+K/V, computed on the host from the very tensors the GPU consumed, and (b) size-independent
+properties: softmax mass conservation through an indicator V (every key counted exactly once),
+constant-V fixed point, and linearity in V.  bf16 bar: max-abs <= 2e-2, cosine >= 0.9999;
+fp8 / sparse-fp8 bar: cosine >= 0.995 against the oracle's fake-quant emulation."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+D = 128
+HEADS_CHECKED = [0, 11, 23]
+
+
+def _sample_rows(S, n=40, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    fixed = [0, 1, 31, 32, 63, 64, 255, 256, S // 2, S - 65, S - 64, S - 41, S - 40, S - 2, S - 1]
+    rnd = torch.randint(0, S, (n,), generator=g).tolist()
+    return torch.tensor(sorted({r for r in fixed + rnd if 0 <= r < S}))
+
+
+def _oracle_rows(inp, rows, *, tabs=None, tile_map=None, fp8=False, heads=HEADS_CHECKED):
+    from oracle import attention_oracle as O
+
+    hs = torch.tensor(heads)
+    q, k, v = (t[:, :, hs].cpu() for t in (inp.q, inp.k, inp.v))
+    w = torch.ones(D)
+    kw = dict(q_norm_weight=w, k_norm_weight=w, q_rows=rows)
+    if tabs is not None:
+        kw.update(rope_q=tuple(t.cpu().double() for t in tabs), rope_mode=O.ROPE_INTERLEAVED)
+    if inp.key_mask is not None:
+        kw.update(key_mask=inp.key_mask.cpu())
+    if tile_map is not None:
+        kw.update(tile_map=tile_map)
+    if fp8:
+        kw.update(fp8_qk=True)
+    return O.reference_layer(q, k, v, **kw)
+
+
+def _run(inp, **extra):
+    import pika_h3_flex_amd as pk
+
+    ones = torch.ones(D, dtype=torch.float32, device="cuda")
+    opts = dict(q_norm_weight=ones, k_norm_weight=ones, norm_eps=1e-6)
+    tabs = None
+    if inp.position_ids is not None:
+        tabs = pk.rope_tables(inp.position_ids)
+        opts.update(rope_mode=pk.ROPE_INTERLEAVED, rope_q=tabs)
+    if inp.key_mask is not None:
+        opts.update(key_mask=inp.key_mask)
+    opts.update(extra)
+    out = pk.attention(inp.q, inp.k, inp.v, **opts)
+    torch.cuda.synchronize()
+    return out, tabs, opts
+
+
+def _check(out, ref, rows, *, max_abs=2e-2, min_cos=0.9999, label=""):
+    from oracle import attention_oracle as O
+
+    got = out[:, rows.cuda()][:, :, torch.tensor(HEADS_CHECKED).cuda()].cpu()
+    err, cos = O.max_abs_and_cosine(got, ref)
+    print(f"{label}: {rows.numel()} rows x {len(HEADS_CHECKED)} heads: max_abs={err:.3e} cos={cos:.7f}", flush=True)
+    assert torch.isfinite(out.float()).all()
+    assert err <= max_abs and cos >= min_cos
+
+
+@pytest.fixture(scope="module")
+def inp480():
+    from pika_h3_flex_amd import workloads
+
+    return workloads.make("480p", seed=0, device="cuda")
+
+
+def test_480p_sampled_rows(inp480):
+    out, tabs, _ = _run(inp480)
+    rows = _sample_rows(inp480.q.shape[1])
+    _check(out, _oracle_rows(inp480, rows, tabs=tabs), rows, label="480p bf16")
+
+
+def test_480p_mass_conservation_and_linearity(inp480):
+    """V = indicator of (key index mod 128): output[d] is the softmax mass on those keys, so each row
+    of the output sums to 1 iff every key is counted exactly once."""
+    import pika_h3_flex_amd as pk
+    from pika_h3_flex_amd.workloads import AttnInputs
+
+    S, H = inp480.q.shape[1], inp480.q.shape[2]
+    ind = torch.zeros((1, S, 1, D), dtype=torch.bfloat16, device="cuda")
+    ind[0, torch.arange(S), 0, torch.arange(S) % D] = 1.0
+    v_ind = ind.expand(1, S, H, D).contiguous()
+    alt = AttnInputs(inp480.q, inp480.k, v_ind, inp480.position_ids, None, "ind")
+    out, _, opts = _run(alt)
+    mass = out.float().sum(-1)
+    assert float((mass - 1.0).abs().max()) < 1.5e-2, float((mass - 1.0).abs().max())
+    # constant V is a fixed point (up to one bf16 rounding of the normalised sum)
+    vc = inp480.v[:, :1].expand(-1, S, -1, -1).contiguous()
+    outc = pk.attention(inp480.q, inp480.k, vc, **opts)
+    torch.cuda.synchronize()
+    assert float((outc.float() - vc.float()).abs().max()) <= 2.0 ** -7 * float(vc.float().abs().max())
+    # linearity in V
+    o1 = pk.attention(inp480.q, inp480.k, inp480.v, **opts).float()
+    o2 = pk.attention(inp480.q, inp480.k, (inp480.v.float() * 0.5).to(torch.bfloat16), **opts).float()
+    torch.cuda.synchronize()
+    assert float((o1 - 2.0 * o2).abs().max()) < 1e-2
+
+
+def test_480p_fp8(inp480):
+    out, tabs, _ = _run(inp480, fp8_qk=True)
+    rows = _sample_rows(inp480.q.shape[1], n=16)
+    _check(out, _oracle_rows(inp480, rows, tabs=tabs, fp8=True), rows, max_abs=1.0, min_cos=0.995, label="480p fp8 vs fp8 oracle")
+
+
+def test_480p_block_sparse_and_fp8(inp480):
+    import pika_h3_flex_amd as pk
+
+    S = inp480.q.shape[1]
+    tm = pk.local_window_tile_map(S, inp480.tokens_per_frame, window_frames=2, global_fraction=0.10, seed=0)
+    bm = pk.BlockMask.from_dense(tm, device="cuda")
+    rows = _sample_rows(S, n=16)
+    out, tabs, _ = _run(inp480, block_mask=bm)
+    _check(out, _oracle_rows(inp480, rows, tabs=tabs, tile_map=tm), rows, label=f"480p sparse ({float(tm.float().mean()):.3f})")
+    out8, _, _ = _run(inp480, block_mask=bm, fp8_qk=True)
+    _check(out8, _oracle_rows(inp480, rows, tabs=tabs, tile_map=tm, fp8=True), rows, max_abs=1.0, min_cos=0.995, label="480p sparse fp8")
+
+
+def test_joint_and_cross_sampled_rows():
+    from pika_h3_flex_amd import workloads
+
+    joint = workloads.make("joint", seed=1, device="cuda")
+    out, tabs, _ = _run(joint)
+    rows = _sample_rows(joint.q.shape[1], n=24)
+    _check(out, _oracle_rows(joint, rows, tabs=tabs), rows, label="joint video+audio")
+    del joint, out
+    cross = workloads.make("cross", seed=1, device="cuda")
+    n_valid = int(cross.key_mask.sum())
+    assert 60 <= n_valid <= 480
+    out, _, _ = _run(cross)
+    rows = _sample_rows(cross.q.shape[1], n=64)
+    _check(out, _oracle_rows(cross, rows), rows, label=f"text cross-attn ({n_valid}/512 valid)")
+
+
+def test_768p_sampled_rows():
+    from pika_h3_flex_amd import workloads
+
+    inp = workloads.make("768p", seed=2, device="cuda")
+    assert inp.q.shape[1] == 124992
+    out, tabs, _ = _run(inp)
+    rows = _sample_rows(inp.q.shape[1], n=8)
+    _check(out, _oracle_rows(inp, rows, tabs=tabs, heads=HEADS_CHECKED), rows, label="768p bf16")
+
+
+def test_golden_vectors():
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as O
+    from tests import golden_cases
+
+    for name, case in sorted(golden_cases.load().items()):
+        opts = {}
+        if "q_norm_w" in case:
+            opts.update(q_norm_weight=case["q_norm_w"].cuda(), k_norm_weight=case["k_norm_w"].cuda())
+        if "position_ids" in case:
+            opts.update(rope_q=pk.rope_tables(case["position_ids"].cuda()), rope_mode=case["rope_mode"])
+        if "key_mask" in case:
+            opts.update(key_mask=case["key_mask"].cuda())
+        if "tile_map" in case:
+            opts.update(block_mask=pk.BlockMask.from_dense(case["tile_map"], device="cuda"))
+        if case.get("fp8"):
+            opts.update(fp8_qk=True)
+        out = pk.attention(case["q"].cuda(), case["k"].cuda(), case["v"].cuda(), **opts)
+        torch.cuda.synchronize()
+        err, cos = O.max_abs_and_cosine(out.cpu(), case["out"])
+        print(f"golden {name}: max_abs={err:.3e} cos={cos:.7f}", flush=True)
+        if case.get("fp8"):
+            assert cos >= 0.995
+        else:
+            assert err <= 2e-2 and cos >= 0.9999
+
+
+class _Attn(torch.nn.Module):
+    def __init__(self, hidden, heads, kv_dim=None):
+        super().__init__()
+        self.heads = heads
+        self.to_q = torch.nn.Linear(hidden, hidden, bias=False)
+        self.to_k = torch.nn.Linear(kv_dim or hidden, hidden, bias=False)
+        self.to_v = torch.nn.Linear(kv_dim or hidden, hidden, bias=False)
+        self.to_out = torch.nn.ModuleList([torch.nn.Linear(hidden, hidden), torch.nn.Identity()])
+        self.norm_q = torch.nn.RMSNorm(hidden // heads, eps=1e-6)
+        self.norm_k = torch.nn.RMSNorm(hidden // heads, eps=1e-6)
+
+
+def test_processor_self_and_cross():
+    """The processor (module projections -> HIP attention -> to_out) against the same composition
+    with the oracle in the middle."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as O
+
+    torch.manual_seed(0)
+    H, hidden, S = 3, 384, 150
+    attn = _Attn(hidden, H).cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        attn.norm_q.weight.add_(0.1 * torch.randn_like(attn.norm_q.weight))
+    x = torch.randn((1, S, hidden), device="cuda", dtype=torch.bfloat16)
+    pos = torch.cat([pk.video_position_ids(2, 7, 10), pk.audio_position_ids(5)], 0).cuda()
+    proc = pk.PikaH3AttnProcessor()
+    with torch.no_grad():
+        y = proc(attn, x, position_ids=pos)
+        q, k, v = (f(x).view(1, S, H, 128) for f in (attn.to_q, attn.to_k, attn.to_v))
+        ref = O.reference_layer(q.cpu(), k.cpu(), v.cpu(), q_norm_weight=attn.norm_q.weight.float().cpu(),
+                                k_norm_weight=attn.norm_k.weight.float().cpu(), rope_q=O.rope_tables(pos.cpu()),
+                                rope_mode=O.ROPE_INTERLEAVED)
+        yref = attn.to_out[0](ref.to(torch.bfloat16).view(1, S, hidden).cuda())
+    assert y.shape == x.shape
+    assert float((y.float() - yref.float()).abs().max()) < 3e-2
+    # cross-attention with a padding mask, no RoPE
+    attn_c = _Attn(hidden, H, kv_dim=200).cuda().to(torch.bfloat16)
+    enc = torch.randn((1, 64, 200), device="cuda", dtype=torch.bfloat16)
+    mask = (torch.arange(64, device="cuda") < 23)[None, :]
+    with torch.no_grad():
+        y = proc(attn_c, x, encoder_hidden_states=enc, attention_mask=mask)
+        q = attn_c.to_q(x).view(1, S, H, 128)
+        k, v = (f(enc).view(1, 64, H, 128) for f in (attn_c.to_k, attn_c.to_v))
+        ref = O.reference_layer(q.cpu(), k.cpu(), v.cpu(), q_norm_weight=attn_c.norm_q.weight.float().cpu(),
+                                k_norm_weight=attn_c.norm_k.weight.float().cpu(), key_mask=mask.cpu())
+        yref = attn_c.to_out[0](ref.to(torch.bfloat16).view(1, S, hidden).cuda())
+    assert float((y.float() - yref.float()).abs().max()) < 3e-2
