@@ -34,6 +34,8 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-rows", type=int, default=16384, help="query rows of the CPU baseline sample (0 = skip)")
     ap.add_argument("--kernel-iters", type=int, default=10)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 1 GiB device-to-device copy, a kernel of known traffic for scaling profiler byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU over the full local sequence (no sequence-parallel split, "
@@ -79,6 +81,13 @@ def main() -> int:
 
     def step():
         pk.attention(inp.q, inp.k, inp.v, out=out, workspace=ws, **opts)
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
