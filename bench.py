@@ -23,6 +23,9 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}  # MI355X dense MFMA, published
 HBM_PEAK_GBS = 8000.0
+# HBM-side bytes per attention-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00,
+# factors from a 1 GiB copy); figures and commands in profiles/attn_fwd_kernel_480p_bf16.md
+MEASURED_TRAFFIC_BYTES = {"480p": 4.69e9}
 
 
 def main() -> int:
@@ -103,7 +106,7 @@ def main() -> int:
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS["fp8" if fp8 else "bf16"]
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": None, "kernel": "attn_fwd_kernel",
+                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "attn_fwd_kernel",
                 "kernel_ms": round(kernel_ms, 4), "flops_per_launch": flops}
 
     cpu = None
