@@ -5,6 +5,7 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "pkh3_common.h"
@@ -91,6 +92,7 @@ WsPlan plan(const pkh3_attn_args* a) {
   w.idx_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * a->Sk * sizeof(int), 256);
   w.plan_off = off;   if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / 4) * w.nKt * sizeof(int), 256);
   w.plan_cnt_off = off; if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / 4) * sizeof(int), 256);
+  w.kmax_off = off;   off = align_up(off + bh * sizeof(float), 256);
   w.total = off;
   return w;
 }
@@ -120,6 +122,7 @@ void build(const pkh3_attn_args* a, Launch& L) {
   q.cos_t = a->q_rope_cos; q.sin_t = a->q_rope_sin;
   q.out = ws + L.w.q_off; q.out_bh_stride = (int64_t)L.w.nQ64 * L.w.qBlkBytes; q.out_blk_stride = L.w.qBlkBytes;
   q.scale_out = fp8 ? (float*)(ws + L.w.qscale_off) : nullptr; q.fp8 = fp8;
+  q.zero_init = (unsigned*)(ws + L.w.kmax_off);
 
   QkPrologueParams& k = L.kp;
   k = QkPrologueParams{};
@@ -130,6 +133,7 @@ void build(const pkh3_attn_args* a, Launch& L) {
   k.gather_idx = L.idx; k.row_cnt = L.cnt;
   k.out = ws + L.w.kv_off; k.out_bh_stride = (int64_t)L.w.nKt * L.w.kvTileBytes; k.out_blk_stride = L.w.kvTileBytes;
   k.scale_out = fp8 ? (float*)(ws + L.w.kscale_off) : nullptr; k.fp8 = fp8;
+  k.norm_max = (unsigned*)(ws + L.w.kmax_off);
 
   VPrologueParams& v = L.vp;
   v = VPrologueParams{};
@@ -151,6 +155,8 @@ void build(const pkh3_attn_args* a, Launch& L) {
   f.plan_cnt = a->blk_row_ptr ? (const int*)(ws + L.w.plan_cnt_off) : nullptr;
   f.plan_stride = L.w.nKt;
   f.qscale = q.scale_out; f.kscale = k.scale_out; f.fp8 = fp8;
+  f.kmax = (const float*)(ws + L.w.kmax_off);
+  f.force_online = getenv("PKH3_FORCE_ONLINE") != nullptr;
 }
 
 int hip_fail(hipError_t e, const char* what) {

@@ -29,6 +29,7 @@ namespace pkh3 {
 constexpr int kWavesPerWg = 8;
 constexpr int kRing = 3;               // LDS ring depth (tiles)
 constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
+constexpr float kStaticMaxLimit = 48.0f;  // logit bounds up to 2^48 may replace the running max (worst term 2^-96)
 
 #define PKH3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 constexpr int kSgMfma = 0x008, kSgDsRead = 0x100;
@@ -102,7 +103,11 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
 
 // Softmax numerators of w.s, then O^T += V^T P^T.  `c` = softmax scale * log2(e) (times the fp8
 // dequantisation scales of this tile); `lim` = keys of this tile that exist (only read when < 64).
-template <bool FP8>
+// STATIC: w.m holds a per-query upper bound of every logit (|q_i| * max_j |k_j| * c), small enough that
+// exp2(logit - bound) cannot underflow; the running max, its exchange across the half-waves and the
+// O^T rescale are then not needed at all, and the numerators of the first 32 keys do not wait for the
+// second half of S^T.
+template <bool FP8, bool STATIC>
 __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* vbuf, float c, int lim, int lane) {
   const int hh = lane >> 5;
   if (lim < kTileKeys) {
@@ -114,18 +119,21 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
         if (key >= lim) w.s[kb][i] = -INFINITY;
       }
   }
-  float mx = fmaxf(w.s[0][0], w.s[1][0]);
+  float m_new = w.m, alpha = 1.0f;
+  if constexpr (!STATIC) {
+    float mx = fmaxf(w.s[0][0], w.s[1][0]);
 #pragma unroll
-  for (int i = 1; i < 16; ++i) mx = fmaxf(fmaxf(mx, w.s[0][i]), w.s[1][i]);
-  mx = max_across_halves(mx) * c;
-  const float m_new = (mx > w.m + kRescaleSlack) ? mx : w.m;
-  const float alpha = __builtin_amdgcn_exp2f(w.m - m_new);
-  w.m = m_new;
-  if (__any(alpha != 1.0f)) {
+    for (int i = 1; i < 16; ++i) mx = fmaxf(fmaxf(mx, w.s[0][i]), w.s[1][i]);
+    mx = max_across_halves(mx) * c;
+    m_new = (mx > w.m + kRescaleSlack) ? mx : w.m;
+    alpha = __builtin_amdgcn_exp2f(w.m - m_new);
+    w.m = m_new;
+    if (__any(alpha != 1.0f)) {
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < 4; ++db)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) w.o[db][i] *= alpha;
+        for (int i = 0; i < 16; ++i) w.o[db][i] *= alpha;
+    }
   }
   bf16x8 pf[2][2];
   float rsum = 0.f;
@@ -145,7 +153,7 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
       }
       pf[kb][b2] = pk;
     }
-  w.l = w.l * alpha + rsum;
+  w.l = STATIC ? w.l + rsum : w.l * alpha + rsum;
   bf16x8 vg[8];
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
@@ -219,22 +227,60 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
   const float* kscale = FP8 ? p.kscale + (int64_t)bh * p.nKt : nullptr;
   const int tail = sk & (kTileKeys - 1);  // keys in the last tile when it is partial
 
-  int slot = 0;
-  for (int i = 0; i < nt; ++i) {
-    // tiles i and i+1 are in LDS for every wave (own slices: vmcnt, the others': barrier), and every
-    // wave is past tile i-1, whose slot takes tile i+2
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    const char* kbuf = lds[slot];
-    if (i + 2 < nt) dma(entry(i + 2) & 0xffffff, slot == 0 ? kRing - 1 : slot - 1);
-    slot = slot == kRing - 1 ? 0 : slot + 1;
-    const int e = entry(i);
-    const int tile = e & 0xffffff;
-    if (SPARSE && !((e >> 24) & row_bit)) continue;  // wave-uniform: this row-block drops the tile
-    qk_tile<FP8>(w, kbuf, kbuf + kKBytes, lane);
-    const float ct = FP8 ? c * kscale[tile] : c;
-    softmax_pv_tile<FP8>(w, kbuf + kKBytes, ct, (tail && tile == nkt - 1) ? tail : kTileKeys, lane);
+  // Upper bound of this query's logits (log2 domain): |q_i| * max_j |k_j| * c.  When it is small for the
+  // whole wave, exp2(logit - bound) stays a normal fp32 number whatever the data (>= 2^(-2*bound)), so the
+  // bound can stand in for the running max.
+  bool static_max = false;
+  if (nt > 0) {
+    float qn2 = 0.f;
+    if constexpr (!FP8) {
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float x = (float)w.qf[ks][j];
+          qn2 = fmaf(x, x, qn2);
+        }
+    } else {
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4)
+#pragma unroll
+        for (int wd = 0; wd < 4; ++wd) {
+          const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w.q8[c4][wd], false);
+          const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(w.q8[c4][wd], true);
+          qn2 += lo[0] * lo[0] + lo[1] * lo[1] + hi[0] * hi[0] + hi[1] * hi[1];
+        }
+    }
+    qn2 += xhalf(qn2);
+    // margins: K' is rounded to bf16 (fp8: to e4m3, relative step 2^-4) after its norm was taken
+    const float bound = sqrtf(qn2) * p.kmax[bh] * c * (FP8 ? 1.08f : 1.01f);
+    static_max = __all(bound <= kStaticMaxLimit) && !p.force_online;
+    if (static_max) w.m = bound;
   }
+
+  int slot = 0;
+#define PKH3_TILE_LOOP(STATIC)                                                                          \
+  for (int i = 0; i < nt; ++i) {                                                                        \
+    /* tiles i and i+1 are in LDS for every wave (own slices: vmcnt, the others': barrier), and every */ \
+    /* wave is past tile i-1, whose slot takes tile i+2 */                                              \
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
+    __syncthreads();                                                                                    \
+    const char* kbuf = lds[slot];                                                                       \
+    if (i + 2 < nt) dma(entry(i + 2) & 0xffffff, slot == 0 ? kRing - 1 : slot - 1);                     \
+    slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
+    const int e = entry(i);                                                                             \
+    const int tile = e & 0xffffff;                                                                      \
+    if (SPARSE && !((e >> 24) & row_bit)) continue; /* wave-uniform: this row-block drops the tile */   \
+    qk_tile<FP8>(w, kbuf, kbuf + kKBytes, lane);                                                        \
+    const float ct = FP8 ? c * kscale[tile] : c;                                                        \
+    softmax_pv_tile<FP8, STATIC>(w, kbuf + kKBytes, ct, (tail && tile == nkt - 1) ? tail : kTileKeys, lane); \
+  }
+  if (static_max) {
+    PKH3_TILE_LOOP(true)
+  } else {
+    PKH3_TILE_LOOP(false)
+  }
+#undef PKH3_TILE_LOOP
 
   // epilogue: O = O^T / l, bf16, 8-byte stores (4 consecutive d per register group)
   __bf16* ob = (__bf16*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;

@@ -12,7 +12,7 @@ struct WsPlan {
   int nKt;       // 64-key tiles
   int kvTileBytes;  // bytes of one [K tile | V tile] record
   int qBlkBytes;    // bytes of one 64-query block of Q images
-  size_t q_off, kv_off, qscale_off, kscale_off, cnt_off, idx_off, plan_off, plan_cnt_off, total;
+  size_t q_off, kv_off, qscale_off, kscale_off, cnt_off, idx_off, plan_off, plan_cnt_off, kmax_off, total;
 };
 
 // One side (Q or K) of the normalise + rotate + lay-out pass.
@@ -33,6 +33,8 @@ struct QkPrologueParams {
   int out_blk_stride;       // bytes between consecutive 64-row blocks
   float* scale_out;         // fp8: [B*H, nBlk64] dequantisation scales, else null
   int fp8;
+  unsigned* zero_init;      // [B*H] words this launch clears (the later K launch max-reduces into them), or null
+  unsigned* norm_max;       // [B*H] float bits: max row norm after norm+rotation (atomic max), or null
 };
 
 struct VPrologueParams {
@@ -64,6 +66,8 @@ struct FwdParams {
   int plan_stride;          // ints between consecutive query tiles' lists
   const float* qscale;      // [B*H, nQ64]
   const float* kscale;      // [B*H, nKt]
+  const float* kmax;        // [B*H] largest K' row norm
+  int force_online;         // debugging: always keep the running max
   int fp8;
 };
 

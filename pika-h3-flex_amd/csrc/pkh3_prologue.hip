@@ -134,6 +134,22 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
     }
   }
 
+  if (p.zero_init && blk == 0 && lane == 0) p.zero_init[b * p.H + h] = 0u;
+  if (p.norm_max) {
+    // largest row norm of this (batch, head) after norm and rotation: an upper bound for every logit is
+    // |q_i| * max_j |k_j|, which lets the attention kernel drop the running max when the bound is small
+    float nmax = 0.f;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      float ssq = 0.f;
+#pragma unroll
+      for (int i = 0; i < 64; ++i) ssq += x[sub][i] * x[sub][i];
+      ssq += xhalf(ssq);
+      nmax = fmaxf(nmax, ssq);
+    }
+    nmax = sqrtf(wave_max(nmax));
+    if (lane == 0) atomicMax(p.norm_max + b * p.H + h, __float_as_uint(nmax));  // non-negative floats order like uints
+  }
   char* ob = p.out + (int64_t)(b * p.H + h) * p.out_bh_stride + (int64_t)blk * p.out_blk_stride;
   if constexpr (!FP8) {
 #pragma unroll
