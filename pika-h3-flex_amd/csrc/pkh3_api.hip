@@ -81,12 +81,9 @@ WsPlan plan(const pkh3_attn_args* a) {
   w.nQ64 = (int)align_up((size_t)(a->Sq + 63) / 64, 4);
   w.nKt = (a->Sk + 63) / 64;
   w.kvTileBytes = (fp8 ? kK8TileBytes : kKTileBytes) + kVTileBytes;
-  w.qBlkBytes = fp8 ? 2 * kQ8BlkBytes : 2 * kQBlkBytes;
   const size_t bh = (size_t)a->B * a->H;
   size_t off = 0;
-  w.q_off = off;      off = align_up(off + bh * w.nQ64 * w.qBlkBytes, 256);
   w.kv_off = off;     off = align_up(off + bh * w.nKt * (size_t)w.kvTileBytes, 256);
-  w.qscale_off = off; if (fp8) off = align_up(off + bh * w.nQ64 * sizeof(float), 256);
   w.kscale_off = off; if (fp8) off = align_up(off + bh * w.nKt * sizeof(float), 256);
   w.cnt_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * sizeof(int), 256);
   w.idx_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * a->Sk * sizeof(int), 256);
@@ -99,7 +96,7 @@ WsPlan plan(const pkh3_attn_args* a) {
 
 struct Launch {
   WsPlan w;
-  QkPrologueParams qp, kp;
+  QkPrologueParams kp;
   VPrologueParams vp;
   FwdParams f;
   int* cnt;
@@ -113,16 +110,6 @@ void build(const pkh3_attn_args* a, Launch& L) {
   L.cnt = a->key_mask ? (int*)(ws + L.w.cnt_off) : nullptr;
   L.idx = a->key_mask ? (int*)(ws + L.w.idx_off) : nullptr;
   const int kBytes = fp8 ? kK8TileBytes : kKTileBytes;
-
-  QkPrologueParams& q = L.qp;
-  q = QkPrologueParams{};
-  q.x = a->q; q.sb = a->q_sb; q.ss = a->q_ss; q.sh = a->q_sh;
-  q.B = a->B; q.H = a->H; q.S = a->Sq; q.nBlk64 = L.w.nQ64;
-  q.norm_w = a->q_norm_w; q.eps = a->norm_eps; q.rope_mode = a->rope_mode;
-  q.cos_t = a->q_rope_cos; q.sin_t = a->q_rope_sin;
-  q.out = ws + L.w.q_off; q.out_bh_stride = (int64_t)L.w.nQ64 * L.w.qBlkBytes; q.out_blk_stride = L.w.qBlkBytes;
-  q.scale_out = fp8 ? (float*)(ws + L.w.qscale_off) : nullptr; q.fp8 = fp8;
-  q.zero_init = (unsigned*)(ws + L.w.kmax_off);
 
   QkPrologueParams& k = L.kp;
   k = QkPrologueParams{};
@@ -141,10 +128,13 @@ void build(const pkh3_attn_args* a, Launch& L) {
   v.B = a->B; v.H = a->H; v.S = a->Sk; v.nKt = L.w.nKt;
   v.gather_idx = L.idx; v.row_cnt = L.cnt;
   v.out = ws + L.w.kv_off + kBytes; v.out_bh_stride = k.out_bh_stride; v.out_tile_stride = L.w.kvTileBytes;
+  v.zero_init = (unsigned*)(ws + L.w.kmax_off);
 
   FwdParams& f = L.f;
   f = FwdParams{};
-  f.qp = ws + L.w.q_off; f.q_bh_stride = q.out_bh_stride; f.q_blk_stride = L.w.qBlkBytes;
+  f.q = a->q; f.q_sb = a->q_sb; f.q_ss = a->q_ss; f.q_sh = a->q_sh;
+  f.q_norm_w = a->q_norm_w; f.q_eps = a->norm_eps; f.q_rope_mode = a->rope_mode;
+  f.q_cos = a->q_rope_cos; f.q_sin = a->q_rope_sin;
   f.kv = ws + L.w.kv_off; f.kv_bh_stride = k.out_bh_stride; f.kv_tile_stride = L.w.kvTileBytes;
   f.row_cnt = L.cnt;
   f.o = a->o; f.o_sb = a->o_sb; f.o_ss = a->o_ss; f.o_sh = a->o_sh;
@@ -154,7 +144,7 @@ void build(const pkh3_attn_args* a, Launch& L) {
   f.plan = a->blk_row_ptr ? (const int*)(ws + L.w.plan_off) : nullptr;
   f.plan_cnt = a->blk_row_ptr ? (const int*)(ws + L.w.plan_cnt_off) : nullptr;
   f.plan_stride = L.w.nKt;
-  f.qscale = q.scale_out; f.kscale = k.scale_out; f.fp8 = fp8;
+  f.kscale = k.scale_out; f.fp8 = fp8;
   f.kmax = (const float*)(ws + L.w.kmax_off);
   f.force_online = getenv("PKH3_FORCE_ONLINE") != nullptr;
 }
@@ -174,9 +164,9 @@ int run_prologue(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
                                 L.w.nKt, (int*)(ws + L.w.plan_cnt_off), st)) != hipSuccess)
       return hip_fail(e, "sparse plan");
   }
-  if ((e = launch_qk_prologue(L.qp, st)) != hipSuccess) return hip_fail(e, "q prologue");
-  if ((e = launch_qk_prologue(L.kp, st)) != hipSuccess) return hip_fail(e, "k prologue");
+  // V first: it also clears the per-head slots the K pass max-reduces its row norms into
   if ((e = launch_v_prologue(L.vp, st)) != hipSuccess) return hip_fail(e, "v prologue");
+  if ((e = launch_qk_prologue(L.kp, st)) != hipSuccess) return hip_fail(e, "k prologue");
   return PKH3_OK;
 }
 

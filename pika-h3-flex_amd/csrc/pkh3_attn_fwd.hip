@@ -201,21 +201,56 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
   auto entry = [&](int i) { return SPARSE ? __builtin_amdgcn_readfirstlane(plan[i]) : i; };
 
   WaveState<FP8> w;
-  float qscale = 1.0f;
   if (nt > 0) {
     dma(entry(0) & 0xffffff, 0);
     if (nt > 1) dma(entry(1) & 0xffffff, 1);
-    const char* qsrc = p.qp + (int64_t)bh * p.q_bh_stride + (int64_t)(q32 >> 1) * p.q_blk_stride;
+  }
+  // Q load, fused with QK-RMSNorm, rotation and (fp8) quantisation: lane (l%32, hh) reads the 64 elements
+  // d = 16*ks + 8*hh + j of query row q32*32 + l%32 -- the ones it carries in the MFMA B images -- so the
+  // operand images are formed in registers and Q' never exists in memory.
+  float qscale = 1.0f;
+  float qn2 = 0.f;  // squared norm of the (rounded / dequantised) Q' row: this lane's half, then the full row
+  {
+    const int qrow = q32 * 32 + (lane & 31);
+    const bool valid = qrow < p.Sq;
+    float x[64];
+    load_row(x, (const __bf16*)p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh + (int64_t)(valid ? qrow : 0) * p.q_ss, valid, hh);
+    const RowTransform tf{p.q_norm_w, p.q_eps, p.q_rope_mode, p.q_cos, p.q_sin};
+    norm_rope_row(x, tf, qrow, valid, hh);
     if constexpr (!FP8) {
-      const bf16x8* qs = (const bf16x8*)qsrc + (q32 & 1) * 8 * 64;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) w.qf[ks] = qs[ks * 64 + lane];
+      for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const __bf16 r = (__bf16)x[ks * 8 + j];
+          w.qf[ks][j] = r;
+          qn2 = fmaf((float)r, (float)r, qn2);
+        }
     } else {
-      const i32x4* qs = (const i32x4*)qsrc + (q32 & 1) * 4 * 64;
+      // one absmax scale per 64-query block = this wave and its neighbour (wave ^ 1)
+      __shared__ float q_amax[kWavesPerWg];
+      float amax = 0.f;
 #pragma unroll
-      for (int c4 = 0; c4 < 4; ++c4) w.q8[c4] = qs[c4 * 64 + lane];
-      qscale = p.qscale[(int64_t)bh * p.nQ64 + (q32 >> 1)];
+      for (int i = 0; i < 64; ++i) amax = fmaxf(amax, fabsf(x[i]));
+      amax = wave_max(amax);
+      if (lane == 0) q_amax[wave] = amax;
+      __syncthreads();
+      amax = fmaxf(amax, q_amax[wave ^ 1]);
+      qscale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
+      const float inv = 1.0f / qscale;
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        w.q8[c4] = quant_fp8_chunk(x, c4, inv);
+#pragma unroll
+        for (int wd = 0; wd < 4; ++wd) {
+          const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w.q8[c4][wd], false);
+          const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(w.q8[c4][wd], true);
+          qn2 += lo[0] * lo[0] + lo[1] * lo[1] + hi[0] * hi[0] + hi[1] * hi[1];
+        }
+      }
+      qn2 *= qscale * qscale;
     }
+    qn2 += xhalf(qn2);
   }
 #pragma unroll
   for (int db = 0; db < 4; ++db)
@@ -232,28 +267,8 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
   // bound can stand in for the running max.
   bool static_max = false;
   if (nt > 0) {
-    float qn2 = 0.f;
-    if constexpr (!FP8) {
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float x = (float)w.qf[ks][j];
-          qn2 = fmaf(x, x, qn2);
-        }
-    } else {
-#pragma unroll
-      for (int c4 = 0; c4 < 4; ++c4)
-#pragma unroll
-        for (int wd = 0; wd < 4; ++wd) {
-          const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w.q8[c4][wd], false);
-          const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(w.q8[c4][wd], true);
-          qn2 += lo[0] * lo[0] + lo[1] * lo[1] + hi[0] * hi[0] + hi[1] * hi[1];
-        }
-    }
-    qn2 += xhalf(qn2);
     // margins: K' is rounded to bf16 (fp8: to e4m3, relative step 2^-4) after its norm was taken
-    const float bound = sqrtf(qn2) * p.kmax[bh] * c * (FP8 ? 1.08f : 1.01f);
+    const float bound = sqrtf(qn2) * p.kmax[bh] * p.c * (FP8 ? 1.08f : 1.01f);
     static_max = __all(bound <= kStaticMaxLimit) && !p.force_online;
     if (static_max) w.m = bound;
   }

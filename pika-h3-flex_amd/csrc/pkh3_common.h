@@ -56,4 +56,94 @@ __device__ __forceinline__ float wave_max(float x) {
   return x;
 }
 
+// RMSNorm + rotation of one row, shared by the K prologue and the attention kernel's Q load.
+// `x` holds this lane's 64 elements d = 16*ks + 8*hh + j (index ks*8 + j) of the row; lane l^32 holds
+// the other 64, so the sum of squares needs one exchange and both pairings of the rotation
+// (interleaved (2i,2i+1) / half-split (i,i+64)) stay inside the lane.
+struct RowTransform {
+  const float* norm_w;  // [D] or null
+  float eps;
+  int rope_mode;        // 0 none, 1 interleaved, 2 half-split
+  const float* cos_t;   // [rows, D/2]
+  const float* sin_t;
+};
+
+// `row` must be readable even when !valid (callers point it at row 0); the values are then zeroed.
+__device__ __forceinline__ void load_row(float (&x)[64], const __bf16* row, bool valid, int hh) {
+  bf16x8 t[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) t[ks] = *(const bf16x8*)(row + 16 * ks + 8 * hh);
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[ks * 8 + j] = valid ? (float)t[ks][j] : 0.f;
+}
+
+__device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform& t, int64_t table_row, bool valid,
+                                              int hh) {
+  if (t.norm_w) {
+    float ssq = 0.f;
+#pragma unroll
+    for (int i = 0; i < 64; ++i) ssq += x[i] * x[i];
+    ssq += xhalf(ssq);
+    const float rs = rsqrtf(ssq * (1.0f / kD) + t.eps);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const f32x4 w0 = *(const f32x4*)(t.norm_w + 16 * ks + 8 * hh);
+      const f32x4 w1 = *(const f32x4*)(t.norm_w + 16 * ks + 8 * hh + 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[ks * 8 + j] *= rs * w0[j];
+        x[ks * 8 + 4 + j] *= rs * w1[j];
+      }
+    }
+  }
+  if (t.rope_mode == 1 && valid) {
+    // interleaved pairs (2i, 2i+1): pair index 8*ks + 4*hh + jj for this lane's elements 2jj, 2jj+1
+    const float* ct = t.cos_t + table_row * (kD / 2);
+    const float* st = t.sin_t + table_row * (kD / 2);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const f32x4 c = *(const f32x4*)(ct + 8 * ks + 4 * hh);
+      const f32x4 s = *(const f32x4*)(st + 8 * ks + 4 * hh);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const float a0 = x[ks * 8 + 2 * jj], a1 = x[ks * 8 + 2 * jj + 1];
+        x[ks * 8 + 2 * jj] = a0 * c[jj] - a1 * s[jj];
+        x[ks * 8 + 2 * jj + 1] = a1 * c[jj] + a0 * s[jj];
+      }
+    }
+  } else if (t.rope_mode == 2 && valid) {
+    // half-split pairs (i, i + 64): element d < 64 of this lane sits at ks < 4, its partner at ks + 4
+    const float* ct = t.cos_t + table_row * (kD / 2);
+    const float* st = t.sin_t + table_row * (kD / 2);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const f32x4 c0 = *(const f32x4*)(ct + 16 * ks + 8 * hh), c1 = *(const f32x4*)(ct + 16 * ks + 8 * hh + 4);
+      const f32x4 s0 = *(const f32x4*)(st + 16 * ks + 8 * hh), s1 = *(const f32x4*)(st + 16 * ks + 8 * hh + 4);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float cj = j < 4 ? c0[j & 3] : c1[j & 3], sj = j < 4 ? s0[j & 3] : s1[j & 3];
+        const float lo = x[ks * 8 + j], hi = x[(ks + 4) * 8 + j];
+        x[ks * 8 + j] = lo * cj - hi * sj;
+        x[(ks + 4) * 8 + j] = hi * cj + lo * sj;
+      }
+    }
+  }
+}
+
+// values 16*c .. 16*c+15 of a lane's row -> one 16-byte chunk of an fp8 e4m3 image
+__device__ __forceinline__ i32x4 quant_fp8_chunk(const float (&x)[64], int c, float inv) {
+  i32x4 t;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const int e = 16 * c + 4 * w;
+    int v = 0;
+    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[e] * inv, x[e + 1] * inv, v, false);
+    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[e + 2] * inv, x[e + 3] * inv, v, true);
+    t[w] = v;
+  }
+  return t;
+}
+
 }  // namespace pkh3

@@ -4,6 +4,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "pkh3_common.h"
+
 namespace pkh3 {
 
 // Where each intermediate lives inside the caller's workspace (byte offsets, 256-aligned).
@@ -11,8 +13,7 @@ struct WsPlan {
   int nQ64;      // 64-query blocks, padded to a multiple of 4 (one workgroup = 4 waves x 64 queries)
   int nKt;       // 64-key tiles
   int kvTileBytes;  // bytes of one [K tile | V tile] record
-  int qBlkBytes;    // bytes of one 64-query block of Q images
-  size_t q_off, kv_off, qscale_off, kscale_off, cnt_off, idx_off, plan_off, plan_cnt_off, kmax_off, total;
+  size_t kv_off, kscale_off, cnt_off, idx_off, plan_off, plan_cnt_off, kmax_off, total;
 };
 
 // One side (Q or K) of the normalise + rotate + lay-out pass.
@@ -33,7 +34,6 @@ struct QkPrologueParams {
   int out_blk_stride;       // bytes between consecutive 64-row blocks
   float* scale_out;         // fp8: [B*H, nBlk64] dequantisation scales, else null
   int fp8;
-  unsigned* zero_init;      // [B*H] words this launch clears (the later K launch max-reduces into them), or null
   unsigned* norm_max;       // [B*H] float bits: max row norm after norm+rotation (atomic max), or null
 };
 
@@ -46,12 +46,17 @@ struct VPrologueParams {
   char* out;                // points at the V part of tile 0
   int64_t out_bh_stride;
   int out_tile_stride;
+  unsigned* zero_init;      // [B*H] words this launch clears (the K launch after it max-reduces into them)
 };
 
 struct FwdParams {
-  const char* qp;           // Q images
-  int64_t q_bh_stride;      // bytes
-  int q_blk_stride;         // bytes per 64-query block
+  const void* q;            // bf16 [B,Sq,H,D] strided; norm + rotation (+ fp8 quantisation) happen at load
+  int64_t q_sb, q_ss, q_sh;
+  const float* q_norm_w;    // RMSNorm weight of the Q side or null
+  float q_eps;
+  int q_rope_mode;
+  const float* q_cos;
+  const float* q_sin;
   const char* kv;           // [K tile | V tile] records
   int64_t kv_bh_stride;
   int kv_tile_stride;
@@ -64,8 +69,7 @@ struct FwdParams {
   const int* plan;          // block-sparse: per query tile (256 queries) the union tile list, or null
   const int* plan_cnt;      // [nQ64/4] entries per query tile
   int plan_stride;          // ints between consecutive query tiles' lists
-  const float* qscale;      // [B*H, nQ64]
-  const float* kscale;      // [B*H, nKt]
+  const float* kscale;      // [B*H, nKt] fp8 dequantisation scales of the K tiles
   const float* kmax;        // [B*H] largest K' row norm
   int force_online;         // debugging: always keep the running max
   int fp8;

@@ -51,7 +51,8 @@ hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int
 }
 
 // ------------------------------------------------------------------------------------------------
-// RMSNorm + RoPE (+ fp8 quantisation) of Q or K rows into operand images.
+// RMSNorm + RoPE (+ fp8 quantisation) of K rows into operand images (the Q side does the same math
+// inside the attention kernel, on the rows each wave owns).
 // One wave owns one 64-row block of one (batch, head): lane (r = l%32, hh = l/32) holds, for the
 // two 32-row halves `sub`, the 64 elements d = 16*ks + 8*hh + j of row 32*sub + r -- exactly the
 // elements its lane carries in the MFMA images, so norm, rotation and the store need one
@@ -66,6 +67,7 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
   const int rows = p.row_cnt ? p.row_cnt[b] : p.S;
   const __bf16* xb = (const __bf16*)p.x + (int64_t)b * p.sb + (int64_t)h * p.sh;
 
+  const RowTransform tf{p.norm_w, p.eps, p.rope_mode, p.cos_t, p.sin_t};
   float x[2][64];
 #pragma unroll
   for (int sub = 0; sub < 2; ++sub) {
@@ -73,68 +75,10 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
     const bool valid = row < rows;
     int src = 0;
     if (valid) src = p.gather_idx ? p.gather_idx[(int64_t)b * p.S + row] : row;
-    const __bf16* xr = xb + (int64_t)src * p.ss;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      bf16x8 t = {};
-      if (valid) t = *(const bf16x8*)(xr + 16 * ks + 8 * hh);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) x[sub][ks * 8 + j] = (float)t[j];
-    }
-    if (p.norm_w) {
-      float ssq = 0.f;
-#pragma unroll
-      for (int i = 0; i < 64; ++i) ssq += x[sub][i] * x[sub][i];
-      ssq += xhalf(ssq);
-      const float rs = rsqrtf(ssq * (1.0f / kD) + p.eps);
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const f32x4 w0 = *(const f32x4*)(p.norm_w + 16 * ks + 8 * hh);
-        const f32x4 w1 = *(const f32x4*)(p.norm_w + 16 * ks + 8 * hh + 4);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          x[sub][ks * 8 + j] *= rs * w0[j];
-          x[sub][ks * 8 + 4 + j] *= rs * w1[j];
-        }
-      }
-    }
-    if (p.rope_mode == 1 && valid) {
-      // interleaved pairs (2i, 2i+1): pair index 8*ks + 4*hh + jj for this lane's elements 2jj, 2jj+1
-      const float* ct = p.cos_t + (int64_t)src * (kD / 2);
-      const float* st = p.sin_t + (int64_t)src * (kD / 2);
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const f32x4 c = *(const f32x4*)(ct + 8 * ks + 4 * hh);
-        const f32x4 s = *(const f32x4*)(st + 8 * ks + 4 * hh);
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          const float a0 = x[sub][ks * 8 + 2 * jj], a1 = x[sub][ks * 8 + 2 * jj + 1];
-          x[sub][ks * 8 + 2 * jj] = a0 * c[jj] - a1 * s[jj];
-          x[sub][ks * 8 + 2 * jj + 1] = a1 * c[jj] + a0 * s[jj];
-        }
-      }
-    } else if (p.rope_mode == 2 && valid) {
-      // half-split pairs (i, i + 64): element d < 64 of this lane sits at ks < 4, its partner at ks + 4
-      const float* ct = p.cos_t + (int64_t)src * (kD / 2);
-      const float* st = p.sin_t + (int64_t)src * (kD / 2);
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-#pragma unroll
-        for (int q4 = 0; q4 < 2; ++q4) {
-          const f32x4 c = *(const f32x4*)(ct + 16 * ks + 8 * hh + 4 * q4);
-          const f32x4 s = *(const f32x4*)(st + 16 * ks + 8 * hh + 4 * q4);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float lo = x[sub][ks * 8 + 4 * q4 + j], hi = x[sub][(ks + 4) * 8 + 4 * q4 + j];
-            x[sub][ks * 8 + 4 * q4 + j] = lo * c[j] - hi * s[j];
-            x[sub][(ks + 4) * 8 + 4 * q4 + j] = hi * c[j] + lo * s[j];
-          }
-        }
-      }
-    }
+    load_row(x[sub], xb + (int64_t)src * p.ss, valid, hh);
+    norm_rope_row(x[sub], tf, src, valid, hh);
   }
 
-  if (p.zero_init && blk == 0 && lane == 0) p.zero_init[b * p.H + h] = 0u;
   if (p.norm_max) {
     // largest row norm of this (batch, head) after norm and rotation: an upper bound for every logit is
     // |q_i| * max_j |k_j|, which lets the attention kernel drop the running max when the bound is small
@@ -174,18 +118,8 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        i32x4 t;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const float* e = &x[sub][c * 16 + w * 4];
-          int v = 0;
-          v = __builtin_amdgcn_cvt_pk_fp8_f32(e[0] * inv, e[1] * inv, v, false);
-          v = __builtin_amdgcn_cvt_pk_fp8_f32(e[2] * inv, e[3] * inv, v, true);
-          t[w] = v;
-        }
-        *(i32x4*)(ob + ((sub * 4 + c) * 64 + lane) * 16) = t;
-      }
+      for (int c = 0; c < 4; ++c)
+        *(i32x4*)(ob + ((sub * 4 + c) * 64 + lane) * 16) = quant_fp8_chunk(x[sub], c, inv);
   }
 }
 
@@ -209,6 +143,7 @@ __global__ __launch_bounds__(256) void v_prologue_kernel(VPrologueParams p) {
   if (t >= p.nKt) return;
   const int h = blockIdx.y, b = blockIdx.z;
   const int r = lane & 31, hh = lane >> 5;
+  if (t == 0 && lane == 0) p.zero_init[b * p.H + h] = 0u;
   const int rows = p.row_cnt ? p.row_cnt[b] : p.S;
   const __bf16* vb = (const __bf16*)p.v + (int64_t)b * p.sb + (int64_t)h * p.sh;
   char* ob = p.out + (int64_t)(b * p.H + h) * p.out_bh_stride + (int64_t)t * p.out_tile_stride;
