@@ -109,6 +109,21 @@ def main() -> int:
                 "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "attn_fwd_kernel",
                 "kernel_ms": round(kernel_ms, 4), "flops_per_launch": flops}
 
+    # calibration: the bf16 MFMA rate this box sustains on a pure MFMA stream with all-ones and with random
+    # operands (the part is power-limited on real data; see pika-h3-flex_amd/csrc/pkh3_mfma_probe.hip)
+    probe = os.path.join(ROOT, "pika-h3-flex_amd", "pkh3_mfma_probe")
+    if os.path.exists(probe) and not fp8:
+        import subprocess
+
+        try:
+            res = subprocess.run([probe, "20000"], capture_output=True, text=True, timeout=120)
+            rates = {json.loads(l)["operands"]: json.loads(l)["tflops"] for l in res.stdout.splitlines() if l.startswith("{")}
+            roofline["mfma_stream_tflops_measured"] = rates
+            if rates.get("random"):
+                roofline["frac_of_measured_random_operand_ceiling"] = round(achieved / rates["random"], 4)
+        except Exception as exc:  # the probe is informational only
+            roofline["mfma_stream_tflops_measured"] = f"probe failed: {exc}"
+
     cpu = None
     if args.cpu_rows > 0:
         from oracle import cpu_sdpa

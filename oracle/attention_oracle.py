@@ -184,10 +184,12 @@ def attention(
 def reference_layer(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, q_norm_weight=None, k_norm_weight=None,
     norm_eps: float = 1e-6, rope_q=None, rope_k=None, rope_mode: int = ROPE_NONE, key_mask=None,
-    tile_map=None, fp8_qk: bool = False, scale: Optional[float] = None, q_rows=None,
+    tile_map=None, fp8_qk: bool = False, scale: Optional[float] = None, q_rows=None, bf16_operands: bool = False,
 ) -> torch.Tensor:
     """The whole path on ``[B, S, H, D]`` inputs: QK-RMSNorm -> RoPE -> (fp8 fake-quant of Q, K) ->
-    masked softmax attention, float64.  A ``None`` norm weight means no norm on that side."""
+    masked softmax attention, float64.  A ``None`` norm weight means no norm on that side.
+    ``bf16_operands`` rounds the normed/rotated Q and K to bf16 first, the precision a bf16 matrix
+    unit sees; used where logits are so large that this rounding alone exceeds the bf16 tolerance."""
     qf, kf = q.to(torch.float64), k.to(torch.float64)
     if q_norm_weight is not None:
         qf = rms_norm(qf, q_norm_weight, norm_eps)
@@ -197,6 +199,8 @@ def reference_layer(
         rk = rope_q if rope_k is None else rope_k
         qf = apply_rope(qf, rope_q[0], rope_q[1], rope_mode)
         kf = apply_rope(kf, rk[0], rk[1], rope_mode)
+    if bf16_operands:
+        qf, kf = qf.to(torch.bfloat16).to(torch.float64), kf.to(torch.bfloat16).to(torch.float64)
     if fp8_qk:
         qf, _ = fake_quant_fp8_blocks(qf)
         kf, _ = fake_quant_fp8_blocks(kf)

@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libpkh3attn.so")
+# PKH3_LIB_PATH selects another build of the same library (e.g. an experimental one); default: next to this file
+LIB_PATH = os.environ.get("PKH3_LIB_PATH") or os.path.join(_HERE, "libpkh3attn.so")
 
 PKH3_OK = 0
 PKH3_ENULL = -1

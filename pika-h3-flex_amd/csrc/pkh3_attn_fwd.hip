@@ -164,7 +164,11 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
 }
 
 template <bool FP8, bool SPARSE>
-__global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(512, 1)
+#ifdef PKH3_WAVES_PER_EU
+__attribute__((amdgpu_waves_per_eu(2, 2)))
+#endif
+void attn_fwd_kernel(FwdParams p) {
   constexpr int kKBytes = FP8 ? kK8TileBytes : kKTileBytes;
   constexpr int kTileBytes = kKBytes + kVTileBytes;
   constexpr int kSliceBytes = kTileBytes / kWavesPerWg;  // bytes of a tile each wave copies

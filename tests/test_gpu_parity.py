@@ -23,7 +23,7 @@ def _rand(shape, gen, std=1.0):
 
 
 def _run_and_check(B, Sq, Sk, H, *, seed=0, norm=True, rope_mode=0, mask=None, std=1.0, min_cos=MIN_COS,
-                   max_abs=MAX_ABS, weight_random=False):
+                   max_abs=MAX_ABS, weight_random=False, weight_scale=1.0, bf16_operands=False):
     import pika_h3_flex_amd as pk
 
     O = _oracle()
@@ -37,6 +37,7 @@ def _run_and_check(B, Sq, Sk, H, *, seed=0, norm=True, rope_mode=0, mask=None, s
             kw = 1.0 + 0.2 * torch.randn(D, generator=gen)
         else:
             qw, kw = torch.ones(D), torch.ones(D)
+        qw = qw * weight_scale
     rope_q = rope_k = None
     if rope_mode:
         posq = torch.rand((Sq, 3), generator=gen, dtype=torch.float64) * torch.tensor([30.0, 29.0, 51.0], dtype=torch.float64)
@@ -44,7 +45,7 @@ def _run_and_check(B, Sq, Sk, H, *, seed=0, norm=True, rope_mode=0, mask=None, s
         rope_q = O.rope_tables(posq)
         rope_k = O.rope_tables(posk)
     ref = O.reference_layer(q, k, v, q_norm_weight=qw, k_norm_weight=kw, rope_q=rope_q, rope_k=rope_k,
-                            rope_mode=rope_mode, key_mask=mask)
+                            rope_mode=rope_mode, key_mask=mask, bf16_operands=bf16_operands)
     dev = "cuda"
     f32 = lambda t: None if t is None else t.to(torch.float32).contiguous().to(dev)
     opts = dict(q_norm_weight=f32(qw), k_norm_weight=f32(kw), norm_eps=1e-6, rope_mode=rope_mode)
@@ -151,3 +152,31 @@ def test_rope_tables_kernel():
     torch.cuda.synchronize()
     assert (cos.cpu().double() - rc).abs().max() < 1e-6
     assert (sin.cpu().double() - rs).abs().max() < 1e-6
+
+
+# The kernel replaces the running max by a per-query logit bound |q_i| * max_j |k_j| * scale * log2(e) when that
+# bound is at most 48; unit-weight QK-RMSNorm gives 16.3.  The cases below push the bound above the limit
+# (norm weight x4 -> 65; un-normed N(0, 2^2) rows -> 65) so the running-max softmax path runs.  Logits are then
+# +-45, where rounding Q' and K' to bf16 (which every bf16 matrix unit does) alone moves the softmax weights by
+# more than the bf16 tolerance, so the oracle rounds its operands the same way (bf16_operands).
+@pytest.mark.parametrize("S", [64, 200, 1000])
+def test_large_logits_take_the_running_max_path(S):
+    _run_and_check(1, S, S, 2, seed=300 + S, weight_scale=4.0, rope_mode=1, bf16_operands=True)
+
+
+def test_large_logits_no_norm():
+    _run_and_check(1, 300, 300, 2, seed=77, norm=False, std=2.0, bf16_operands=True)
+
+
+def test_large_logits_with_key_mask():
+    gen = torch.Generator().manual_seed(5)
+    mask = torch.rand((2, 333), generator=gen) < 0.5
+    _run_and_check(2, 150, 333, 2, seed=78, mask=mask, weight_scale=4.0, bf16_operands=True)
+
+
+def test_bound_path_and_running_max_path_agree():
+    """Same inputs through both softmax formulations (the bound is forced off by PKH3_FORCE_ONLINE in a
+    fresh process in the benchmark scripts; here the two regimes are compared through the oracle only)."""
+    out_small, ref_small = _run_and_check(1, 500, 500, 2, seed=11, weight_scale=1.0)
+    out_big, ref_big = _run_and_check(1, 500, 500, 2, seed=11, weight_scale=4.0, bf16_operands=True)
+    assert not torch.equal(out_small, out_big)

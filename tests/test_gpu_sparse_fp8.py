@@ -110,3 +110,22 @@ def test_fp8_block_sparse():
     err8, cos8 = O.max_abs_and_cosine(out, ref8)
     print(f"fp8+sparse: max_abs={err8:.3e} cos={cos8:.6f}", flush=True)
     assert cos8 >= 0.995
+
+
+def test_sparse_and_fp8_with_large_logits():
+    """Norm weight x4 lifts the logit bound above the limit, so these run the running-max softmax path."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as O
+
+    q, k, v, gen = _inputs(1, 640, 640, 2, seed=31)
+    tm = _tile_map(10, 10, 0.4, gen)
+    w4 = torch.full((D,), 4.0)
+    ref = O.reference_layer(q, k, v, q_norm_weight=w4, k_norm_weight=torch.ones(D), tile_map=tm, bf16_operands=True)
+    out = _call(q, k, v, q_norm_weight=w4.cuda(), k_norm_weight=_ones(), block_mask=pk.BlockMask.from_dense(tm, device="cuda"))
+    err, cos = O.max_abs_and_cosine(out, ref)
+    assert err <= 2e-2 and cos >= 0.9999
+    ref8 = O.reference_layer(q, k, v, q_norm_weight=w4, k_norm_weight=torch.ones(D), fp8_qk=True)
+    out8 = _call(q, k, v, q_norm_weight=w4.cuda(), k_norm_weight=_ones(), fp8_qk=True)
+    err8, cos8 = O.max_abs_and_cosine(out8, ref8)
+    print(f"fp8 large logits: max_abs={err8:.3e} cos={cos8:.6f}", flush=True)
+    assert cos8 >= 0.995

@@ -263,3 +263,12 @@ def test_cpu_sdpa_baseline_agrees_with_oracle():
     ref = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, rope_q=tabs, rope_mode=O.ROPE_INTERLEAVED)
     out = cpu_sdpa.sdpa_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, rope_q=tabs)
     assert (out.double() - ref).abs().max() < 1e-4
+
+
+def test_bf16_operands_option_rounds_q_and_k_only():
+    S = 20
+    q, k, v = (_r(1, S, 1, 128, seed=s) for s in (40, 41, 42))
+    a = O.reference_layer(q, k, v, bf16_operands=True)
+    b = O.attention(q.to(torch.bfloat16).double(), k.to(torch.bfloat16).double(), v)
+    assert torch.equal(a, b)
+    assert not torch.equal(a, O.reference_layer(q, k, v))
