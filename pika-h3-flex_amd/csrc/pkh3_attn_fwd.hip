@@ -18,9 +18,10 @@
 // The transposed formulation keeps every per-query quantity (max, sum, rescale factor) a per-lane
 // scalar: no cross-lane traffic in the rescale, none between the two GEMMs.
 //
-// Block-sparse variant.  The 4 query row-blocks (64 queries each, two waves per row-block) of a
-// workgroup walk the union of their tile lists; a wave skips the math of a tile its row-block does
-// not keep.  The union list (tile index + 4-bit row mask) is built on the device by a plan kernel.
+// Block-sparse variant.  A workgroup covers 4 query row-blocks (64 queries each, a wave pair per row-block).
+// Phase 1 walks the key tiles all four row-blocks keep, exactly like the dense kernel.  Phase 2 walks the
+// remaining tiles per row-block: every iteration gives each wave pair one 32-key half of a tile of its own
+// list in its own LDS area, so all 8 waves stay busy.  The lists are built on the device by a plan kernel.
 #include "pkh3_common.h"
 #include "pkh3_internal.h"
 
@@ -32,12 +33,24 @@ constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when ex
 constexpr float kStaticMaxLimit = 48.0f;  // logit bounds up to 2^48 may replace the running max (worst term 2^-96)
 
 #define PKH3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+// Each tile loop ends on an 8-pass MFMA into the O^T accumulators.  The compiler was seen to place the register
+// copies that merge the two loop variants (v_mov_b64 reading the accumulator's last registers) four scalar
+// instructions after that MFMA, before its result is written back; the block-sparse kernel then returned a stale
+// O^T block.  32 idle issue cycles after every loop let the last MFMA retire whatever follows.
+#define PKH3_MFMA_DRAIN() asm volatile("s_nop 15\n\ts_nop 15" ::: "memory")
 constexpr int kSgMfma = 0x008, kSgDsRead = 0x100;
 
 __device__ __forceinline__ void lds_dma16(const char* g, char* l) {
   // 64 lanes x 16 B, global -> LDS without passing through VGPRs; LDS address = l + lane*16
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
                                    (__attribute__((address_space(3))) void*)l, 16, 0, 0);
+}
+
+// Wave-uniform reads of tables earlier kernels wrote (tile lists, fp8 scales): through the scalar cache, so
+// they count on lgkmcnt and never make the wave wait for its outstanding HBM->LDS copies (vmcnt).
+template <typename T>
+__device__ __forceinline__ T uniform_load(const T* p, int i) {
+  return ((const __attribute__((address_space(4))) T*)p)[i];
 }
 
 __device__ __forceinline__ float max_across_halves(float x) {
@@ -163,16 +176,97 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
   }
 }
 
+// ---- 32-key half tiles, used by the second phase of the block-sparse kernel -----------------------------
+// S^T (32 keys x 32 queries) into w.s[0]; kbuf/vbuf point at this half's K images (8 bf16 / 4 fp8 chunks)
+// and V images (8).
+template <bool FP8>
+__device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) w.s[0][i] = 0.f;
+  if constexpr (!FP8) {
+    bf16x8 kf[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      w.s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], w.qf[i], w.s[0], 0, 0, 0);
+      w.vf[i] = *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
+    }
+  } else {
+    i32x4 kc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) kc[i] = *(const i32x4*)(kbuf + (i * 64 + lane) * 16);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const i32x4 a0 = kc[2 * ks], a1 = kc[2 * ks + 1];
+      const i32x4 b0 = w.q8[2 * ks], b1 = w.q8[2 * ks + 1];
+      const i32x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+      const i32x8 b = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+      w.s[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, w.s[0], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w.vf[4 * ks + i] = *(const bf16x8*)(vbuf + ((4 * ks + i) * 64 + lane) * 16);
+    }
+  }
+}
+
+// Softmax numerators of w.s[0] and O^T += V^T P^T for one half tile (V images already in w.vf).
+// `lim` = keys of this half that exist (<= 0: none; only read when < 32).
+template <bool FP8, bool STATIC>
+__device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int lim, int lane) {
+  const int hh = lane >> 5;
+  if (lim < 32) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = 8 * (i / 4) + 4 * hh + (i % 4);
+      if (key >= lim) w.s[0][i] = -INFINITY;
+    }
+  }
+  float m_new = w.m, alpha = 1.0f;
+  if constexpr (!STATIC) {
+    float mx = w.s[0][0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, w.s[0][i]);
+    mx = max_across_halves(mx) * c;
+    m_new = (mx > w.m + kRescaleSlack) ? mx : w.m;
+    alpha = __builtin_amdgcn_exp2f(w.m - m_new);
+    w.m = m_new;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) w.o[db][i] *= alpha;
+    }
+  }
+  bf16x8 pf[2];
+  float rsum = 0.f;
+  const bf16x2 one2 = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+  for (int b2 = 0; b2 < 2; ++b2) {
+    bf16x8 pk;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pk[j] = (__bf16)__builtin_amdgcn_exp2f(fmaf(w.s[0][8 * b2 + j], c, -m_new));
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      const bf16x2 pr = {pk[j], pk[j + 1]};
+      rsum = __builtin_amdgcn_fdot2_f32_bf16(pr, one2, rsum, false);
+    }
+    pf[b2] = pk;
+  }
+  w.l = STATIC ? w.l + rsum : w.l * alpha + rsum;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) w.o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w.vf[i], pf[i >> 2], w.o[i & 3], 0, 0, 0);
+}
+
 template <bool FP8, bool SPARSE>
-__global__ __launch_bounds__(512, 1)
-#ifdef PKH3_WAVES_PER_EU
-__attribute__((amdgpu_waves_per_eu(2, 2)))
-#endif
-void attn_fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
   constexpr int kKBytes = FP8 ? kK8TileBytes : kKTileBytes;
   constexpr int kTileBytes = kKBytes + kVTileBytes;
   constexpr int kSliceBytes = kTileBytes / kWavesPerWg;  // bytes of a tile each wave copies
-  __shared__ __attribute__((aligned(1024))) char lds[kRing][kTileBytes];
+  constexpr int kHalfBytes = kTileBytes / 2;  // K and V images of 32 keys
+  // dense / phase 1: ring of kRing whole tiles; sparse phase 2: two stages of four row-private half tiles
+  constexpr int kLdsBytes = SPARSE && 8 * kHalfBytes > kRing * kTileBytes ? 8 * kHalfBytes : kRing * kTileBytes;
+  __shared__ __attribute__((aligned(1024))) char lds_raw[kLdsBytes];
+  char(*lds)[kTileBytes] = (char(*)[kTileBytes])lds_raw;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int hh = lane >> 5;
@@ -190,9 +284,10 @@ void attn_fwd_kernel(FwdParams p) {
 
   const int sk = p.row_cnt ? p.row_cnt[b] : p.Sk;
   const int nkt = (sk + kTileKeys - 1) / kTileKeys;
+  // sparse: [tiles every row-block of this workgroup keeps | tiles only row-block 0 keeps | ... 1 | 2 | 3]
   const int* plan = SPARSE ? p.plan + (int64_t)qt * p.plan_stride : nullptr;
-  const int nt = SPARSE ? p.plan_cnt[qt] : nkt;  // tiles this workgroup walks
-  const int row_bit = 1 << (wave >> 1);          // sparse: this wave's row-block inside the workgroup
+  const int* plan_cnt = SPARSE ? p.plan_cnt + qt * 5 : nullptr;
+  const int nt = SPARSE ? uniform_load(plan_cnt, 0) : nkt;  // tiles all 8 waves walk together
 
   // this wave's slice of every [K|V] tile record
   const char* kv_w = p.kv + (int64_t)bh * p.kv_bh_stride + wave * kSliceBytes + lane * 16;
@@ -202,12 +297,12 @@ void attn_fwd_kernel(FwdParams p) {
 #pragma unroll
     for (int i = 0; i < kSliceBytes / 1024; ++i) lds_dma16(g + i * 1024, d + i * 1024);
   };
-  auto entry = [&](int i) { return SPARSE ? __builtin_amdgcn_readfirstlane(plan[i]) : i; };
+  auto entry = [&](int i) { return SPARSE ? uniform_load(plan, i) : i; };  // i-th shared tile
 
   WaveState<FP8> w;
   if (nt > 0) {
-    dma(entry(0) & 0xffffff, 0);
-    if (nt > 1) dma(entry(1) & 0xffffff, 1);
+    dma(entry(0), 0);
+    if (nt > 1) dma(entry(1), 1);
   }
   // Q load, fused with QK-RMSNorm, rotation and (fp8) quantisation: lane (l%32, hh) reads the 64 elements
   // d = 16*ks + 8*hh + j of query row q32*32 + l%32 -- the ones it carries in the MFMA B images -- so the
@@ -272,7 +367,7 @@ void attn_fwd_kernel(FwdParams p) {
   bool static_max = false;
   if (nt > 0) {
     // margins: K' is rounded to bf16 (fp8: to e4m3, relative step 2^-4) after its norm was taken
-    const float bound = sqrtf(qn2) * p.kmax[bh] * p.c * (FP8 ? 1.08f : 1.01f);
+    const float bound = sqrtf(qn2) * uniform_load(p.kmax, bh) * p.c * (FP8 ? 1.08f : 1.01f);
     static_max = __all(bound <= kStaticMaxLimit) && !p.force_online;
     if (static_max) w.m = bound;
   }
@@ -285,21 +380,71 @@ void attn_fwd_kernel(FwdParams p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
     __syncthreads();                                                                                    \
     const char* kbuf = lds[slot];                                                                       \
-    if (i + 2 < nt) dma(entry(i + 2) & 0xffffff, slot == 0 ? kRing - 1 : slot - 1);                     \
+    if (i + 2 < nt) dma(entry(i + 2), slot == 0 ? kRing - 1 : slot - 1);                                \
     slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
-    const int e = entry(i);                                                                             \
-    const int tile = e & 0xffffff;                                                                      \
-    if (SPARSE && !((e >> 24) & row_bit)) continue; /* wave-uniform: this row-block drops the tile */   \
+    const int tile = entry(i);                                                                          \
     qk_tile<FP8>(w, kbuf, kbuf + kKBytes, lane);                                                        \
-    const float ct = FP8 ? c * kscale[tile] : c;                                                        \
+    const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
     softmax_pv_tile<FP8, STATIC>(w, kbuf + kKBytes, ct, (tail && tile == nkt - 1) ? tail : kTileKeys, lane); \
   }
   if (static_max) {
     PKH3_TILE_LOOP(true)
+    PKH3_MFMA_DRAIN();
   } else {
     PKH3_TILE_LOOP(false)
+    PKH3_MFMA_DRAIN();
   }
 #undef PKH3_TILE_LOOP
+
+  if constexpr (SPARSE) {
+    // Phase 2: the tiles that only some row-blocks keep.  Each row-block (a wave pair) walks its own list in
+    // 32-key halves; an iteration gives every pair one half tile in its own LDS area, so all 8 waves stay
+    // busy whichever rows a tile belongs to.  Two stages, the next half tile is copied while this one is used.
+    const int r = wave >> 1;  // row-block of this wave inside the workgroup
+    const int* mine = plan + (1 + r) * p.nKt;
+    const int n_mine = uniform_load(plan_cnt, 1 + r);
+    const int n_iter = 2 * max(max(uniform_load(plan_cnt, 1), uniform_load(plan_cnt, 2)),
+                               max(uniform_load(plan_cnt, 3), uniform_load(plan_cnt, 4)));
+    constexpr int kKHalf = kKBytes / 2, kVHalf = kVTileBytes / 2;
+    // this wave copies half of its pair's K half (and V half): K images are 1 KiB x (8 bf16 | 4 fp8) per half
+    auto dma_half = [&](int it, int stage) {
+      const int tile = uniform_load(mine, it >> 1);
+      const int kb = it & 1;
+      const char* g = p.kv + (int64_t)bh * p.kv_bh_stride + (int64_t)tile * p.kv_tile_stride + lane * 16;
+      char* d = lds_raw + (stage * 4 + r) * kHalfBytes;
+      const int sub = wave & 1;
+#pragma unroll
+      for (int i = 0; i < kKHalf / 2048; ++i)
+        lds_dma16(g + kb * kKHalf + (sub * (kKHalf / 2048) + i) * 1024, d + (sub * (kKHalf / 2048) + i) * 1024);
+#pragma unroll
+      for (int i = 0; i < kVHalf / 2048; ++i)
+        lds_dma16(g + kKBytes + kb * kVHalf + (sub * (kVHalf / 2048) + i) * 1024,
+                  d + kKHalf + (sub * (kVHalf / 2048) + i) * 1024);
+    };
+    __syncthreads();  // every wave is done with the phase-1 ring
+    if (n_mine > 0) dma_half(0, 0);
+#define PKH3_HALF_LOOP(STATIC)                                                                          \
+  for (int it = 0; it < n_iter; ++it) {                                                                 \
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
+    __syncthreads();                                                                                    \
+    if (it + 1 < 2 * n_mine) dma_half(it + 1, (it + 1) & 1);                                            \
+    if (it >= 2 * n_mine) continue; /* wave-uniform: this row-block has run out of tiles */             \
+    const int tile = uniform_load(mine, it >> 1);                                                       \
+    const char* hbuf = lds_raw + ((it & 1) * 4 + r) * kHalfBytes;                                       \
+    qk_half<FP8>(w, hbuf, hbuf + kKHalf, lane);                                                         \
+    const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
+    const int lim = (tail && tile == nkt - 1) ? tail - 32 * (it & 1) : 32;                              \
+    softmax_pv_half<FP8, STATIC>(w, ct, lim, lane);                                                     \
+  }
+    if (static_max) {
+      PKH3_HALF_LOOP(true)
+      PKH3_MFMA_DRAIN();
+    } else {
+      PKH3_HALF_LOOP(false)
+      PKH3_MFMA_DRAIN();
+    }
+#undef PKH3_HALF_LOOP
+  }
 
   // epilogue: O = O^T / l, bf16, 8-byte stores (4 consecutive d per register group)
   __bf16* ob = (__bf16*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
@@ -340,9 +485,10 @@ hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Block-sparse plan: for each workgroup (4 consecutive 64-query row-blocks) the ascending list of key
-// tiles any of its row-blocks keeps, each entry = tile index | (row mask << 24).  One workgroup per
-// query tile merges the four CSR rows through an LDS mask array, walking the key tiles in chunks.
+// Block-sparse plan.  For each workgroup (4 consecutive 64-query row-blocks) five ascending tile lists, each
+// `nKt` ints apart: [0] the key tiles every one of its row-blocks keeps (walked by all 8 waves together),
+// [1+r] the tiles row-block r keeps that are not in [0] (walked by that row-block's wave pair).  One
+// workgroup per query tile merges the four CSR rows through an LDS mask array, key tiles in chunks.
 constexpr int kPlanChunk = 8192;
 
 __global__ __launch_bounds__(256) void sparse_plan_kernel(const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
@@ -350,41 +496,44 @@ __global__ __launch_bounds__(256) void sparse_plan_kernel(const int* __restrict_
                                                           int* __restrict__ plan_cnt) {
   __shared__ unsigned char mask[kPlanChunk];
   __shared__ int wave_tot[4];
-  __shared__ int carry;
+  __shared__ int carry[5];
   const int qt = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int* out = plan + (int64_t)qt * plan_stride;
-  if (tid == 0) carry = 0;
+  const int rows_here = min(4, nRow64 - qt * 4);
+  const int full = (1 << rows_here) - 1;
+  if (tid < 5) carry[tid] = 0;
   for (int base = 0; base < nKt; base += kPlanChunk) {
     for (int i = tid; i < kPlanChunk; i += 256) mask[i] = 0;
     __syncthreads();
-    for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < rows_here; ++r) {
       const int row = qt * 4 + r;
-      if (row < nRow64) {
-        const int beg = row_ptr[row], end = row_ptr[row + 1];
-        for (int j = beg + tid; j < end; j += 256) {
-          const int col = col_idx[j] - base;
-          // a row lists a column at most once, so within one r no two threads touch the same byte
-          if (col >= 0 && col < kPlanChunk && col + base < nKt) mask[col] |= (unsigned char)(1 << r);
-        }
+      const int beg = row_ptr[row], end = row_ptr[row + 1];
+      for (int j = beg + tid; j < end; j += 256) {
+        const int col = col_idx[j] - base;
+        // a row lists a column at most once, so within one r no two threads touch the same byte
+        if (col >= 0 && col < kPlanChunk && col + base < nKt) mask[col] |= (unsigned char)(1 << r);
       }
       __syncthreads();
     }
-    for (int c0 = 0; c0 < kPlanChunk && base + c0 < nKt; c0 += 256) {
-      const int col = c0 + tid;
-      const int mk = (base + col < nKt) ? mask[col] : 0;
-      const unsigned long long bal = __ballot(mk != 0);
-      const int before = __popcll(bal & ((1ull << lane) - 1ull));
-      if (lane == 0) wave_tot[wave] = __popcll(bal);
-      __syncthreads();
-      int off = carry;
-      for (int wv = 0; wv < wave; ++wv) off += wave_tot[wv];
-      if (mk) out[off + before] = (base + col) | (mk << 24);
-      __syncthreads();
-      if (tid == 0) carry += wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
-      __syncthreads();
+    for (int list = 0; list < 5; ++list) {
+      for (int c0 = 0; c0 < kPlanChunk && base + c0 < nKt; c0 += 256) {
+        const int col = c0 + tid;
+        const int mk = (base + col < nKt) ? mask[col] : 0;
+        const bool take = list == 0 ? (mk == full && full != 0) : (((mk >> (list - 1)) & 1) && mk != full);
+        const unsigned long long bal = __ballot(take);
+        const int before = __popcll(bal & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_tot[wave] = __popcll(bal);
+        __syncthreads();
+        int off = carry[list];
+        for (int wv = 0; wv < wave; ++wv) off += wave_tot[wv];
+        if (take) out[list * nKt + off + before] = base + col;
+        __syncthreads();
+        if (tid == 0) carry[list] += wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
+        __syncthreads();
+      }
     }
   }
-  if (tid == 0) plan_cnt[qt] = carry;
+  if (tid < 5) plan_cnt[qt * 5 + tid] = carry[tid];
 }
 
 hipError_t launch_sparse_plan(const int* row_ptr, const int* col_idx, int nRow64, int nQ64, int nKt, int* plan,

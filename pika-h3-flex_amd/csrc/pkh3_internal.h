@@ -66,9 +66,9 @@ struct FwdParams {
   int B, H, Sq, Sk;
   int nQ64, nKt;
   float c;                  // softmax_scale * log2(e)
-  const int* plan;          // block-sparse: per query tile (256 queries) the union tile list, or null
-  const int* plan_cnt;      // [nQ64/4] entries per query tile
-  int plan_stride;          // ints between consecutive query tiles' lists
+  const int* plan;          // block-sparse: per query tile (256 queries) five tile lists nKt ints apart, or null
+  const int* plan_cnt;      // [nQ64/4][5] entries per list
+  int plan_stride;          // ints between consecutive query tiles' lists (5 * nKt)
   const float* kscale;      // [B*H, nKt] fp8 dequantisation scales of the K tiles
   const float* kmax;        // [B*H] largest K' row norm
   int force_online;         // debugging: always keep the running max
