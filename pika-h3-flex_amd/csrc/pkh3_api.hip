@@ -5,7 +5,6 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
-#include <stdlib.h>
 #include <string.h>
 
 #include "pkh3_common.h"
@@ -146,7 +145,6 @@ void build(const pkh3_attn_args* a, Launch& L) {
   f.plan_stride = 5 * L.w.nKt;
   f.kscale = k.scale_out; f.fp8 = fp8;
   f.kmax = (const float*)(ws + L.w.kmax_off);
-  f.force_online = getenv("PKH3_FORCE_ONLINE") != nullptr;
 }
 
 int hip_fail(hipError_t e, const char* what) {

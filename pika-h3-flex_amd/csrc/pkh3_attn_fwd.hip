@@ -1,11 +1,13 @@
 // Non-causal flash-style attention forward for gfx950 (CDNA4), head dim 128.
 //
-// Work split.  A workgroup is 8 waves, two per SIMD; each wave owns 32 queries of one (batch, head)
-// and keeps for them, in VGPRs, the Q operand images, the running row max / row sum and the fp32
-// output accumulator O^T (128 x 32).  The 8 waves share every 64-key K/V tile, which is copied
-// HBM/L2 -> LDS with direct-to-LDS loads into a 3-slot ring, two tiles ahead of the math.  Two waves
-// per SIMD is what overlaps the softmax VALU work of one wave with the MFMAs of the other; the whole
-// per-wave state stays under 256 VGPRs so no accumulator ever moves between register files.
+// Work split.  A workgroup is 12 waves (dense; three per SIMD) or 8 waves (block-sparse; two per SIMD);
+// each wave owns 32 queries of one (batch, head) and keeps for them, in VGPRs, the Q operand images, the
+// running row max / row sum and the fp32 output accumulator O^T (128 x 32).  All waves share every 64-key
+// K/V tile, which is copied HBM/L2 -> LDS with direct-to-LDS loads into a 3-slot ring, two tiles ahead of
+// the math.  Several waves per SIMD is what overlaps the softmax VALU work of one wave with the MFMAs of
+// another; the whole per-wave state stays in VGPRs (<= 168 dense, <= 256 sparse) so no accumulator ever
+// moves between register files.  Q is read in place: RMSNorm, rotation and fp8 quantisation of the Q rows
+// happen in registers while the first K/V tiles are in flight.
 //
 // Math per tile, all on the 32x32 MFMA shapes (see pkh3_common.h for the operand images):
 //   S^T = K' Q'^T      A = K image (LDS), B = Q image (VGPR)      -> lane l holds query l%32, 16 keys / block
@@ -27,7 +29,8 @@
 
 namespace pkh3 {
 
-constexpr int kWavesPerWg = 8;
+constexpr int kDenseWaves = 12;  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
+constexpr int kSparseWaves = 8;  // the block-sparse kernel is built around 4 row-blocks x 2 waves (two per SIMD)
 constexpr int kRing = 3;               // LDS ring depth (tiles)
 constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
 constexpr float kStaticMaxLimit = 48.0f;  // logit bounds up to 2^48 may replace the running max (worst term 2^-96)
@@ -70,13 +73,30 @@ struct WaveState {
 
 // S^T = K' Q'^T for the 64 keys of one tile.  LDS reads run 8 images ahead of the MFMAs that consume
 // them; the tail of the MFMA chain covers the first V image reads.
-template <bool FP8>
+// LEAN (three waves per SIMD, 168 VGPRs): the reads run only 4 images ahead and V is left to the P.V loop.
+template <bool FP8, bool LEAN>
 __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane) {
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
     for (int i = 0; i < 16; ++i) w.s[kb][i] = 0.f;
-  if constexpr (!FP8) {
+  if constexpr (!FP8 && LEAN) {
+    bf16x8 kf[16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int kb = i >> 3, ks = i & 7;
+      w.s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], w.qf[ks], w.s[kb], 0, 0, 0);
+      if (i + 4 < 16) kf[i + 4] = *(const bf16x8*)(kbuf + ((i + 4) * 64 + lane) * 16);
+    }
+    PKH3_SGB(kSgDsRead, 4);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      PKH3_SGB(kSgMfma, 1);
+      if (i + 4 < 16) PKH3_SGB(kSgDsRead, 1);
+    }
+  } else if constexpr (!FP8) {
     bf16x8 kf[16];
 #pragma unroll
     for (int i = 0; i < 8; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
@@ -120,7 +140,7 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
 // exp2(logit - bound) cannot underflow; the running max, its exchange across the half-waves and the
 // O^T rescale are then not needed at all, and the numerators of the first 32 keys do not wait for the
 // second half of S^T.
-template <bool FP8, bool STATIC>
+template <bool FP8, bool STATIC, bool LEAN>
 __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* vbuf, float c, int lim, int lane) {
   const int hh = lane >> 5;
   if (lim < kTileKeys) {
@@ -167,12 +187,24 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
       pf[kb][b2] = pk;
     }
   w.l = STATIC ? w.l + rsum : w.l * alpha + rsum;
-  bf16x8 vg[8];
+  if constexpr (!FP8 && LEAN) {
+    bf16x8 vg[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int kb = i >> 3, b2 = (i >> 2) & 1, db = i & 3;
-    w.o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(i < 8 ? w.vf[i] : vg[i - 8], pf[kb][b2], w.o[db], 0, 0, 0);
-    if (i < 8) vg[i] = *(const bf16x8*)(vbuf + ((i + 8) * 64 + lane) * 16);
+    for (int i = 0; i < 4; ++i) vg[i] = *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int kb = i >> 3, b2 = (i >> 2) & 1, db = i & 3;
+      w.o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vg[i], pf[kb][b2], w.o[db], 0, 0, 0);
+      if (i + 4 < 16) vg[i + 4] = *(const bf16x8*)(vbuf + ((i + 4) * 64 + lane) * 16);
+    }
+  } else {
+    bf16x8 vg[8];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int kb = i >> 3, b2 = (i >> 2) & 1, db = i & 3;
+      w.o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(i < 8 ? w.vf[i] : vg[i - 8], pf[kb][b2], w.o[db], 0, 0, 0);
+      if (i < 8) vg[i] = *(const bf16x8*)(vbuf + ((i + 8) * 64 + lane) * 16);
+    }
   }
 }
 
@@ -257,11 +289,12 @@ __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int 
   for (int i = 0; i < 8; ++i) w.o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w.vf[i], pf[i >> 2], w.o[i & 3], 0, 0, 0);
 }
 
-template <bool FP8, bool SPARSE>
-__global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
+template <bool FP8, bool SPARSE, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
+  static_assert(!SPARSE || WAVES == kSparseWaves, "block-sparse layout assumes 8 waves per workgroup");
   constexpr int kKBytes = FP8 ? kK8TileBytes : kKTileBytes;
   constexpr int kTileBytes = kKBytes + kVTileBytes;
-  constexpr int kSliceBytes = kTileBytes / kWavesPerWg;  // bytes of a tile each wave copies
+  constexpr int kChunks = kTileBytes / 1024;  // 1 KiB pieces of a tile, dealt round-robin to the waves
   constexpr int kHalfBytes = kTileBytes / 2;  // K and V images of 32 keys
   // dense / phase 1: ring of kRing whole tiles; sparse phase 2: two stages of four row-private half tiles
   constexpr int kLdsBytes = SPARSE && 8 * kHalfBytes > kRing * kTileBytes ? 8 * kHalfBytes : kRing * kTileBytes;
@@ -273,14 +306,14 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
 
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD one contiguous run of
   // (batch, head, query tile) so the 32 CUs behind one L2 stream the same K/V at the same time.
-  const int nQt = p.nQ64 / 4;
+  const int nQt = (p.nQ64 * 2 + WAVES - 1) / WAVES;
   const int total = p.B * p.H * nQt;
   const int per_xcd = (total + 7) / 8;
   const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (lin >= total) return;
   const int bh = lin / nQt, qt = lin % nQt;
   const int b = bh / p.H, h = bh % p.H;
-  const int q32 = qt * kWavesPerWg + wave;  // 32-query block of this wave
+  const int q32 = qt * WAVES + wave;  // 32-query block of this wave
 
   const int sk = p.row_cnt ? p.row_cnt[b] : p.Sk;
   const int nkt = (sk + kTileKeys - 1) / kTileKeys;
@@ -289,13 +322,14 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
   const int* plan_cnt = SPARSE ? p.plan_cnt + qt * 5 : nullptr;
   const int nt = SPARSE ? uniform_load(plan_cnt, 0) : nkt;  // tiles all 8 waves walk together
 
-  // this wave's slice of every [K|V] tile record
-  const char* kv_w = p.kv + (int64_t)bh * p.kv_bh_stride + wave * kSliceBytes + lane * 16;
+  // this wave's pieces of every [K|V] tile record: 1 KiB chunks wave, wave + WAVES, ...
+  const char* kv_w = p.kv + (int64_t)bh * p.kv_bh_stride + wave * 1024 + lane * 16;
   auto dma = [&](int tile, int slot) {
     const char* g = kv_w + (int64_t)tile * p.kv_tile_stride;
-    char* d = lds[slot] + wave * kSliceBytes;
+    char* d = lds[slot] + wave * 1024;
 #pragma unroll
-    for (int i = 0; i < kSliceBytes / 1024; ++i) lds_dma16(g + i * 1024, d + i * 1024);
+    for (int i = 0; i < (kChunks + WAVES - 1) / WAVES; ++i)
+      if (i * WAVES + wave < kChunks) lds_dma16(g + i * WAVES * 1024, d + i * WAVES * 1024);
   };
   auto entry = [&](int i) { return SPARSE ? uniform_load(plan, i) : i; };  // i-th shared tile
 
@@ -327,7 +361,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
         }
     } else {
       // one absmax scale per 64-query block = this wave and its neighbour (wave ^ 1)
-      __shared__ float q_amax[kWavesPerWg];
+      __shared__ float q_amax[WAVES];
       float amax = 0.f;
 #pragma unroll
       for (int i = 0; i < 64; ++i) amax = fmaxf(amax, fabsf(x[i]));
@@ -368,7 +402,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
   if (nt > 0) {
     // margins: K' is rounded to bf16 (fp8: to e4m3, relative step 2^-4) after its norm was taken
     const float bound = sqrtf(qn2) * uniform_load(p.kmax, bh) * p.c * (FP8 ? 1.08f : 1.01f);
-    static_max = __all(bound <= kStaticMaxLimit) && !p.force_online;
+    static_max = __all(bound <= kStaticMaxLimit);
     if (static_max) w.m = bound;
   }
 
@@ -383,9 +417,9 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
     if (i + 2 < nt) dma(entry(i + 2), slot == 0 ? kRing - 1 : slot - 1);                                \
     slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
     const int tile = entry(i);                                                                          \
-    qk_tile<FP8>(w, kbuf, kbuf + kKBytes, lane);                                                        \
+    qk_tile<FP8, (WAVES > 8)>(w, kbuf, kbuf + kKBytes, lane);                                           \
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
-    softmax_pv_tile<FP8, STATIC>(w, kbuf + kKBytes, ct, (tail && tile == nkt - 1) ? tail : kTileKeys, lane); \
+    softmax_pv_tile<FP8, STATIC, (WAVES > 8)>(w, kbuf + kKBytes, ct, (tail && tile == nkt - 1) ? tail : kTileKeys, lane); \
   }
   if (static_max) {
     PKH3_TILE_LOOP(true)
@@ -465,21 +499,21 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_kernel(FwdParams p) {
   }
 }
 
-hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
-  const int nQt = p.nQ64 / 4;
+template <bool FP8, bool SPARSE, int WAVES>
+static void launch_variant(const FwdParams& p, hipStream_t st) {
+  const int nQt = (p.nQ64 * 2 + WAVES - 1) / WAVES;
   const int total = p.B * p.H * nQt;
-  const dim3 grid((total + 7) / 8 * 8), block(64 * kWavesPerWg);
+  hipLaunchKernelGGL((attn_fwd_kernel<FP8, SPARSE, WAVES>), dim3((total + 7) / 8 * 8), dim3(64 * WAVES), 0, st, p);
+}
+
+hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
   const bool sparse = p.plan != nullptr;
   if (p.fp8) {
-    if (sparse)
-      hipLaunchKernelGGL((attn_fwd_kernel<true, true>), grid, block, 0, st, p);
-    else
-      hipLaunchKernelGGL((attn_fwd_kernel<true, false>), grid, block, 0, st, p);
+    if (sparse) launch_variant<true, true, kSparseWaves>(p, st);
+    else launch_variant<true, false, kDenseWaves>(p, st);
   } else {
-    if (sparse)
-      hipLaunchKernelGGL((attn_fwd_kernel<false, true>), grid, block, 0, st, p);
-    else
-      hipLaunchKernelGGL((attn_fwd_kernel<false, false>), grid, block, 0, st, p);
+    if (sparse) launch_variant<false, true, kSparseWaves>(p, st);
+    else launch_variant<false, false, kDenseWaves>(p, st);
   }
   return hipGetLastError();
 }

@@ -71,7 +71,6 @@ struct FwdParams {
   int plan_stride;          // ints between consecutive query tiles' lists (5 * nKt)
   const float* kscale;      // [B*H, nKt] fp8 dequantisation scales of the K tiles
   const float* kmax;        // [B*H] largest K' row norm
-  int force_online;         // debugging: always keep the running max
   int fp8;
 };
 
