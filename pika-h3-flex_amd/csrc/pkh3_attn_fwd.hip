@@ -29,7 +29,11 @@
 
 namespace pkh3 {
 
-constexpr int kDenseWaves = 12;  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
+#ifdef PKH3_X_W8
+constexpr int kDenseWaves = 8;
+#else
+constexpr int kDenseWaves = 12;
+#endif  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
 constexpr int kSparseWaves = 8;  // the block-sparse kernel is built around 4 row-blocks x 2 waves (two per SIMD)
 constexpr int kRing = 3;               // LDS ring depth (tiles)
 constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
@@ -44,9 +48,15 @@ constexpr float kStaticMaxLimit = 48.0f;  // logit bounds up to 2^48 may replace
 constexpr int kSgMfma = 0x008, kSgDsRead = 0x100;
 
 __device__ __forceinline__ void lds_dma16(const char* g, char* l) {
-  // 64 lanes x 16 B, global -> LDS without passing through VGPRs; LDS address = l + lane*16
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                   (__attribute__((address_space(3))) void*)l, 16, 0, 0);
+  // 64 lanes x 16 B, global -> LDS without passing through VGPRs; LDS address = l + lane*16.
+  // Issued through inline assembly on purpose: once the compiler sees a direct-to-LDS load it stops trusting
+  // the in-order LDS counter and turns every later wait on an LDS read into lgkmcnt(0), which serialises the
+  // operand image reads.  Completion is tracked by hand: the s_waitcnt vmcnt(0) at the top of each tile loop.
+  const unsigned lds_addr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)l;
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(g), "s"(lds_addr)
+               : "memory");
 }
 
 // Wave-uniform reads of tables earlier kernels wrote (tile lists, fp8 scales): through the scalar cache, so
@@ -140,10 +150,10 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
 // exp2(logit - bound) cannot underflow; the running max, its exchange across the half-waves and the
 // O^T rescale are then not needed at all, and the numerators of the first 32 keys do not wait for the
 // second half of S^T.
-template <bool FP8, bool STATIC, bool LEAN>
+template <bool FP8, bool STATIC, bool LEAN, bool MASKED>
 __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* vbuf, float c, int lim, int lane) {
   const int hh = lane >> 5;
-  if (lim < kTileKeys) {
+  if constexpr (MASKED) {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -407,8 +417,12 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
   }
 
   int slot = 0;
-#define PKH3_TILE_LOOP(STATIC)                                                                          \
-  for (int i = 0; i < nt; ++i) {                                                                        \
+  // Only the last key tile can be partial.  It is peeled off the loop so that the loop body has no masking
+  // branch between S^T and the softmax, which lets the numerators of the first 32 keys be scheduled under
+  // the MFMAs of the second 32.
+  const int n_masked = (tail && nt > 0 && entry(nt - 1) == nkt - 1) ? 1 : 0;
+#define PKH3_TILE_LOOP(STATIC, MASKED, FROM, TO)                                                        \
+  for (int i = FROM; i < TO; ++i) {                                                                     \
     /* tiles i and i+1 are in LDS for every wave (own slices: vmcnt, the others': barrier), and every */ \
     /* wave is past tile i-1, whose slot takes tile i+2 */                                              \
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
@@ -419,13 +433,15 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
     const int tile = entry(i);                                                                          \
     qk_tile<FP8, (WAVES > 8)>(w, kbuf, kbuf + kKBytes, lane);                                           \
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
-    softmax_pv_tile<FP8, STATIC, (WAVES > 8)>(w, kbuf + kKBytes, ct, (tail && tile == nkt - 1) ? tail : kTileKeys, lane); \
+    softmax_pv_tile<FP8, STATIC, (WAVES > 8), MASKED>(w, kbuf + kKBytes, ct, tail, lane);                 \
   }
   if (static_max) {
-    PKH3_TILE_LOOP(true)
+    PKH3_TILE_LOOP(true, false, 0, nt - n_masked)
+    PKH3_TILE_LOOP(true, true, nt - n_masked, nt)
     PKH3_MFMA_DRAIN();
   } else {
-    PKH3_TILE_LOOP(false)
+    PKH3_TILE_LOOP(false, false, 0, nt - n_masked)
+    PKH3_TILE_LOOP(false, true, nt - n_masked, nt)
     PKH3_MFMA_DRAIN();
   }
 #undef PKH3_TILE_LOOP
