@@ -188,8 +188,10 @@ def reference_layer(
 ) -> torch.Tensor:
     """The whole path on ``[B, S, H, D]`` inputs: QK-RMSNorm -> RoPE -> (fp8 fake-quant of Q, K) ->
     masked softmax attention, float64.  A ``None`` norm weight means no norm on that side.
-    ``bf16_operands`` rounds the normed/rotated Q and K to bf16 first, the precision a bf16 matrix
-    unit sees; used where logits are so large that this rounding alone exceeds the bf16 tolerance."""
+    ``bf16_operands`` rounds the normed/rotated K, and the normed/rotated Q times
+    ``scale * log2(e)`` (the factor a log2-domain kernel carries in its Q operand), to bf16 first: the
+    precision a bf16 matrix unit sees.  Used where logits are so large that this rounding alone
+    exceeds the bf16 tolerance."""
     qf, kf = q.to(torch.float64), k.to(torch.float64)
     if q_norm_weight is not None:
         qf = rms_norm(qf, q_norm_weight, norm_eps)
@@ -200,7 +202,9 @@ def reference_layer(
         qf = apply_rope(qf, rope_q[0], rope_q[1], rope_mode)
         kf = apply_rope(kf, rk[0], rk[1], rope_mode)
     if bf16_operands:
-        qf, kf = qf.to(torch.bfloat16).to(torch.float64), kf.to(torch.bfloat16).to(torch.float64)
+        cq = (float(scale) if scale is not None else q.shape[-1] ** -0.5) * math.log2(math.e)
+        qf = (qf * cq).to(torch.bfloat16).to(torch.float64) / cq
+        kf = kf.to(torch.bfloat16).to(torch.float64)
     if fp8_qk:
         qf, _ = fake_quant_fp8_blocks(qf)
         kf, _ = fake_quant_fp8_blocks(kf)

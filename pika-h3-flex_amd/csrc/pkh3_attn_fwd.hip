@@ -29,15 +29,11 @@
 
 namespace pkh3 {
 
-#ifdef PKH3_X_W8
-constexpr int kDenseWaves = 8;
-#else
-constexpr int kDenseWaves = 12;
-#endif  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
+constexpr int kDenseWaves = 12;  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
 constexpr int kSparseWaves = 8;  // the block-sparse kernel is built around 4 row-blocks x 2 waves (two per SIMD)
 constexpr int kRing = 3;               // LDS ring depth (tiles)
 constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
-constexpr float kStaticMaxLimit = 48.0f;  // logit bounds up to 2^48 may replace the running max (worst term 2^-96)
+constexpr float kStaticMaxLimit = 48.0f;  // rows whose |logit| bound is below this skip the running max (terms 2^-48 .. 2^48)
 
 #define PKH3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 // Each tile loop ends on an 8-pass MFMA into the O^T accumulators.  The compiler was seen to place the register
@@ -150,6 +146,15 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
 // exp2(logit - bound) cannot underflow; the running max, its exchange across the half-waves and the
 // O^T rescale are then not needed at all, and the numerators of the first 32 keys do not wait for the
 // second half of S^T.
+// exp2 of one logit.  bf16 path: Q' already carries softmax_scale * log2(e), so S^T is in the log2 domain and
+// `c` is unused; fp8 path: `c` carries that factor times the dequantisation scales.  STATIC: the logits are
+// bounded in magnitude (see kStaticMaxLimit), so no maximum is subtracted at all.
+template <bool FP8, bool STATIC>
+__device__ __forceinline__ float softmax_numerator(float s, float c, float m) {
+  if constexpr (FP8) return __builtin_amdgcn_exp2f(STATIC ? s * c : fmaf(s, c, -m));
+  else return __builtin_amdgcn_exp2f(STATIC ? s : s - m);
+}
+
 template <bool FP8, bool STATIC, bool LEAN, bool MASKED>
 __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* vbuf, float c, int lim, int lane) {
   const int hh = lane >> 5;
@@ -167,7 +172,7 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
     float mx = fmaxf(w.s[0][0], w.s[1][0]);
 #pragma unroll
     for (int i = 1; i < 16; ++i) mx = fmaxf(fmaxf(mx, w.s[0][i]), w.s[1][i]);
-    mx = max_across_halves(mx) * c;
+    mx = max_across_halves(mx) * (FP8 ? c : 1.0f);
     m_new = (mx > w.m + kRescaleSlack) ? mx : w.m;
     alpha = __builtin_amdgcn_exp2f(w.m - m_new);
     w.m = m_new;
@@ -187,7 +192,7 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
     for (int b2 = 0; b2 < 2; ++b2) {
       bf16x8 pk;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) pk[j] = (__bf16)__builtin_amdgcn_exp2f(fmaf(w.s[kb][8 * b2 + j], c, -m_new));
+      for (int j = 0; j < 8; ++j) pk[j] = (__bf16)softmax_numerator<FP8, STATIC>(w.s[kb][8 * b2 + j], c, m_new);
       // row sum over the bf16-rounded values, the same numbers the P.V MFMA consumes
 #pragma unroll
       for (int j = 0; j < 8; j += 2) {
@@ -268,7 +273,7 @@ __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int 
     float mx = w.s[0][0];
 #pragma unroll
     for (int i = 1; i < 16; ++i) mx = fmaxf(mx, w.s[0][i]);
-    mx = max_across_halves(mx) * c;
+    mx = max_across_halves(mx) * (FP8 ? c : 1.0f);
     m_new = (mx > w.m + kRescaleSlack) ? mx : w.m;
     alpha = __builtin_amdgcn_exp2f(w.m - m_new);
     w.m = m_new;
@@ -286,7 +291,7 @@ __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int 
   for (int b2 = 0; b2 < 2; ++b2) {
     bf16x8 pk;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) pk[j] = (__bf16)__builtin_amdgcn_exp2f(fmaf(w.s[0][8 * b2 + j], c, -m_new));
+    for (int j = 0; j < 8; ++j) pk[j] = (__bf16)softmax_numerator<FP8, STATIC>(w.s[0][8 * b2 + j], c, m_new);
 #pragma unroll
     for (int j = 0; j < 8; j += 2) {
       const bf16x2 pr = {pk[j], pk[j + 1]};
@@ -365,7 +370,8 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
       for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const __bf16 r = (__bf16)x[ks * 8 + j];
+          // softmax_scale * log2(e) rides in Q', so S^T comes out of the MFMAs in the log2 domain
+          const __bf16 r = (__bf16)(x[ks * 8 + j] * p.c);
           w.qf[ks][j] = r;
           qn2 = fmaf((float)r, (float)r, qn2);
         }
@@ -405,15 +411,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
   const float* kscale = FP8 ? p.kscale + (int64_t)bh * p.nKt : nullptr;
   const int tail = sk & (kTileKeys - 1);  // keys in the last tile when it is partial
 
-  // Upper bound of this query's logits (log2 domain): |q_i| * max_j |k_j| * c.  When it is small for the
-  // whole wave, exp2(logit - bound) stays a normal fp32 number whatever the data (>= 2^(-2*bound)), so the
-  // bound can stand in for the running max.
+  // Upper bound of the magnitude of this query's logits (log2 domain): |q_i| * max_j |k_j| * c.  When it is
+  // small for the whole wave, exp2(logit) is a normal number in fp32 and in bf16 whatever the data, and so are
+  // the row sums and O^T (at most 2^bound * keys * |v|), so no running max is needed at all.
   bool static_max = false;
   if (nt > 0) {
     // margins: K' is rounded to bf16 (fp8: to e4m3, relative step 2^-4) after its norm was taken
-    const float bound = sqrtf(qn2) * uniform_load(p.kmax, bh) * p.c * (FP8 ? 1.08f : 1.01f);
+    const float bound = sqrtf(qn2) * uniform_load(p.kmax, bh) * (FP8 ? p.c * 1.08f : 1.01f);
     static_max = __all(bound <= kStaticMaxLimit);
-    if (static_max) w.m = bound;
   }
 
   int slot = 0;
