@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per attention-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00,
 # factors from a 1 GiB copy); figures and commands in profiles/attn_fwd_kernel_480p_bf16.md and
 # profiles/attn_fwd_kernel_480p_sparse_fp8.md
-MEASURED_TRAFFIC_BYTES = {"480p": 3.96e9, "480p-sparse-fp8": 2.17e10}
+MEASURED_TRAFFIC_BYTES = {"480p": 3.96e9, "480p-sparse-fp8": 2.11e10}
 
 
 def main() -> int:
@@ -110,20 +110,28 @@ def main() -> int:
                 "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "attn_fwd_kernel",
                 "kernel_ms": round(kernel_ms, 4), "flops_per_launch": flops}
 
-    # calibration: the bf16 MFMA rate this box sustains on a pure MFMA stream with all-ones and with random
-    # operands (the part is power-limited on real data; see pika-h3-flex_amd/csrc/pkh3_mfma_probe.hip)
+    # calibration: what this box sustains on bf16 MFMA work with nothing else in the way -- a pure MFMA stream with
+    # all-ones and with random operands (the part is power-limited on real data), and an attention-shaped tile
+    # loop fed from LDS with no HBM traffic (see pika-h3-flex_amd/csrc/pkh3_mfma_probe.hip)
     probe = os.path.join(ROOT, "pika-h3-flex_amd", "pkh3_mfma_probe")
     if os.path.exists(probe) and not fp8:
         import subprocess
 
         try:
             res = subprocess.run([probe, "20000"], capture_output=True, text=True, timeout=120)
-            rates = {json.loads(l)["operands"]: json.loads(l)["tflops"] for l in res.stdout.splitlines() if l.startswith("{")}
-            roofline["mfma_stream_tflops_measured"] = rates
-            if rates.get("random"):
-                roofline["frac_of_measured_random_operand_ceiling"] = round(achieved / rates["random"], 4)
+            cases = {}
+            for line in res.stdout.splitlines():
+                if line.startswith("{"):
+                    d = json.loads(line)
+                    cases[d["operands"]] = {"tflops": d["tflops"], "core_clock_ghz": d["core_clock_ghz"],
+                                            "mfma_pipe_busy": d["mfma_pipe_busy"]}
+            roofline["mfma_probe"] = cases
+            if cases.get("random"):
+                roofline["frac_of_measured_random_operand_ceiling"] = round(achieved / cases["random"]["tflops"], 4)
+            if cases.get("attention"):
+                roofline["frac_of_attention_shaped_ceiling"] = round(achieved / cases["attention"]["tflops"], 4)
         except Exception as exc:  # the probe is informational only
-            roofline["mfma_stream_tflops_measured"] = f"probe failed: {exc}"
+            roofline["mfma_probe"] = f"probe failed: {exc}"
 
     cpu = None
     if args.cpu_rows > 0:
