@@ -134,8 +134,13 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
       const i32x8 b = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
       // format codes 0/0 = e4m3 x e4m3; scale operands 0 select the unscaled form of the instruction
       w.s[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, w.s[kb], 0, 0, 0, 0, 0, 0);
-      w.vf[2 * i] = *(const bf16x8*)(vbuf + ((2 * i) * 64 + lane) * 16);
-      w.vf[2 * i + 1] = *(const bf16x8*)(vbuf + ((2 * i + 1) * 64 + lane) * 16);
+      // the MFMA chain covers the first V image reads: 8 images, or 4 where registers are short (LEAN)
+      if constexpr (LEAN) {
+        w.vf[i] = *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
+      } else {
+        w.vf[2 * i] = *(const bf16x8*)(vbuf + ((2 * i) * 64 + lane) * 16);
+        w.vf[2 * i + 1] = *(const bf16x8*)(vbuf + ((2 * i + 1) * 64 + lane) * 16);
+      }
     }
   }
 }
@@ -202,10 +207,10 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
       pf[kb][b2] = pk;
     }
   w.l = STATIC ? w.l + rsum : w.l * alpha + rsum;
-  if constexpr (!FP8 && LEAN) {
+  if constexpr (LEAN) {
     bf16x8 vg[16];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) vg[i] = *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
+    for (int i = 0; i < 4; ++i) vg[i] = FP8 ? w.vf[i] : *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int kb = i >> 3, b2 = (i >> 2) & 1, db = i & 3;
