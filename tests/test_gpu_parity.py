@@ -180,3 +180,48 @@ def test_bound_path_and_running_max_path_agree():
     out_small, ref_small = _run_and_check(1, 500, 500, 2, seed=11, weight_scale=1.0)
     out_big, ref_big = _run_and_check(1, 500, 500, 2, seed=11, weight_scale=4.0, bf16_operands=True)
     assert not torch.equal(out_small, out_big)
+
+
+@pytest.mark.parametrize("variant", ["dense_rope_mask", "sparse_fp8"])
+def test_hip_graph_replays_match_eager(variant):
+    """The layer call allocates nothing and only launches kernels on the caller's stream, so it can be captured
+    into a HIP graph.  Every replay, with fresh inputs in the captured buffers and eager work in between, must
+    give the bits of an eager call on the same inputs."""
+    import pika_h3_flex_amd as pk
+
+    B, S, H, D = 1, 333, 2, 128
+    gen = torch.Generator().manual_seed(91)
+    dev = "cuda"
+    q, k, v = (_rand((B, S, H, D), gen).to(dev) for _ in range(3))
+    w = torch.ones(D, device=dev)
+    opts = dict(q_norm_weight=w, k_norm_weight=w)
+    if variant == "dense_rope_mask":
+        pos = torch.rand((S, 3), generator=gen, dtype=torch.float64) * 20.0
+        cos, sin = pk.rope_tables(pos.to(dev))
+        mask = (torch.rand((B, S), generator=gen) < 0.7).to(dev)
+        opts.update(rope_mode=1, rope_q=(cos, sin), key_mask=mask)
+    else:
+        tm = torch.rand((6, 6), generator=gen) < 0.5
+        tm |= torch.eye(6, dtype=torch.bool)
+        opts.update(block_mask=pk.BlockMask.from_dense(tm, device=dev), fp8_qk=True)
+    out = torch.empty_like(q)
+    ws = torch.empty(1 << 22, dtype=torch.uint8, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        pk.attention(q, k, v, out=out, workspace=ws, **opts)  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        pk.attention(q, k, v, out=out, workspace=ws, **opts)
+    for rep in range(4):
+        fresh = [_rand((B, S, H, D), gen).to(dev) for _ in range(3)]
+        eager = pk.attention(*fresh, **opts).clone()
+        torch.cuda.synchronize()
+        for dst, src in zip((q, k, v), fresh):
+            dst.copy_(src)
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager call"
