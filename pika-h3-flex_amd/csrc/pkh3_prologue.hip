@@ -60,9 +60,11 @@ hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int
 template <bool FP8>
 __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int blk = blockIdx.x * 4 + wave;
+  // heads vary fastest across workgroups: neighbouring workgroups then read neighbouring 256-byte pieces of
+  // the same [S, H, D] rows at the same time
+  const int blk = blockIdx.y * 4 + wave;
   if (blk >= p.nBlk64) return;
-  const int h = blockIdx.y, b = blockIdx.z;
+  const int h = blockIdx.x, b = blockIdx.z;
   const int r = lane & 31, hh = lane >> 5;
   const int rows = p.row_cnt ? p.row_cnt[b] : p.S;
   const __bf16* xb = (const __bf16*)p.x + (int64_t)b * p.sb + (int64_t)h * p.sh;
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
 }
 
 hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st) {
-  dim3 grid((p.nBlk64 + 3) / 4, p.H, p.B);
+  dim3 grid(p.H, (p.nBlk64 + 3) / 4, p.B);
   if (p.fp8)
     hipLaunchKernelGGL(qk_prologue_kernel<true>, grid, dim3(256), 0, st, p);
   else
@@ -139,9 +141,9 @@ hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st) {
 // stores are full 1 KiB lines.
 __global__ __launch_bounds__(256) void v_prologue_kernel(VPrologueParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int t = blockIdx.x * 4 + wave;
+  const int t = blockIdx.y * 4 + wave;
   if (t >= p.nKt) return;
-  const int h = blockIdx.y, b = blockIdx.z;
+  const int h = blockIdx.x, b = blockIdx.z;  // heads fastest, as in the K prologue
   const int r = lane & 31, hh = lane >> 5;
   if (t == 0 && lane == 0) p.zero_init[b * p.H + h] = 0u;
   const int rows = p.row_cnt ? p.row_cnt[b] : p.S;
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(256) void v_prologue_kernel(VPrologueParams p) {
 }
 
 hipError_t launch_v_prologue(const VPrologueParams& p, hipStream_t st) {
-  dim3 grid((p.nKt + 3) / 4, p.H, p.B);
+  dim3 grid(p.H, (p.nKt + 3) / 4, p.B);
   hipLaunchKernelGGL(v_prologue_kernel, grid, dim3(256), 0, st, p);
   return hipGetLastError();
 }
