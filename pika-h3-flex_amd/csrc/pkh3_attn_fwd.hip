@@ -43,15 +43,17 @@ constexpr float kStaticMaxLimit = 48.0f;  // rows whose |logit| bound is below t
 #define PKH3_MFMA_DRAIN() asm volatile("s_nop 15\n\ts_nop 15" ::: "memory")
 constexpr int kSgMfma = 0x008, kSgDsRead = 0x100;
 
-__device__ __forceinline__ void lds_dma16(const char* g, char* l) {
-  // 64 lanes x 16 B, global -> LDS without passing through VGPRs; LDS address = l + lane*16.
+__device__ __forceinline__ void lds_dma16(const char* g, unsigned lane_off, char* l) {
+  // 64 lanes x 16 B, global -> LDS without passing through VGPRs: lane i copies g[lane_off_i .. +16) to
+  // l + i*16.  `g` and `l` are wave-uniform (the address arithmetic stays on the scalar unit), `lane_off` is
+  // the per-lane byte offset.
   // Issued through inline assembly on purpose: once the compiler sees a direct-to-LDS load it stops trusting
   // the in-order LDS counter and turns every later wait on an LDS read into lgkmcnt(0), which serialises the
   // operand image reads.  Completion is tracked by hand: the s_waitcnt vmcnt(0) at the top of each tile loop.
   const unsigned lds_addr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)l;
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
-               : "v"(g), "s"(lds_addr)
+               : "v"(lane_off), "s"(g), "s"(lds_addr)
                : "memory");
 }
 
@@ -343,13 +345,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
   const int nt = SPARSE ? uniform_load(plan_cnt, 0) : nkt;  // tiles all 8 waves walk together
 
   // this wave's pieces of every [K|V] tile record: 1 KiB chunks wave, wave + WAVES, ...
-  const char* kv_w = p.kv + (int64_t)bh * p.kv_bh_stride + wave * 1024 + lane * 16;
+  const char* kv_w = p.kv + (int64_t)bh * p.kv_bh_stride + wave * 1024;
+  const unsigned lane_off = lane * 16;
   auto dma = [&](int tile, int slot) {
     const char* g = kv_w + (int64_t)tile * p.kv_tile_stride;
     char* d = lds[slot] + wave * 1024;
 #pragma unroll
     for (int i = 0; i < (kChunks + WAVES - 1) / WAVES; ++i)
-      if (i * WAVES + wave < kChunks) lds_dma16(g + i * WAVES * 1024, d + i * WAVES * 1024);
+      if (i * WAVES + wave < kChunks) lds_dma16(g + i * WAVES * 1024, lane_off, d + i * WAVES * 1024);
   };
   auto entry = [&](int i) { return SPARSE ? uniform_load(plan, i) : i; };  // i-th shared tile
 
@@ -470,15 +473,15 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
     auto dma_half = [&](int it, int stage) {
       const int tile = uniform_load(mine, it >> 1);
       const int kb = it & 1;
-      const char* g = p.kv + (int64_t)bh * p.kv_bh_stride + (int64_t)tile * p.kv_tile_stride + lane * 16;
+      const char* g = p.kv + (int64_t)bh * p.kv_bh_stride + (int64_t)tile * p.kv_tile_stride;
       char* d = lds_raw + (stage * 4 + r) * kHalfBytes;
       const int sub = wave & 1;
 #pragma unroll
       for (int i = 0; i < kKHalf / 2048; ++i)
-        lds_dma16(g + kb * kKHalf + (sub * (kKHalf / 2048) + i) * 1024, d + (sub * (kKHalf / 2048) + i) * 1024);
+        lds_dma16(g + kb * kKHalf + (sub * (kKHalf / 2048) + i) * 1024, lane_off, d + (sub * (kKHalf / 2048) + i) * 1024);
 #pragma unroll
       for (int i = 0; i < kVHalf / 2048; ++i)
-        lds_dma16(g + kKBytes + kb * kVHalf + (sub * (kVHalf / 2048) + i) * 1024,
+        lds_dma16(g + kKBytes + kb * kVHalf + (sub * (kVHalf / 2048) + i) * 1024, lane_off,
                   d + kKHalf + (sub * (kVHalf / 2048) + i) * 1024);
     };
     __syncthreads();  // every wave is done with the phase-1 ring
