@@ -429,7 +429,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
     static_max = __all(bound <= kStaticMaxLimit);
   }
 
-  int slot = 0;
+  int slot = 0, slot_prev = kRing - 1;  // ring slots of tile i and of tile i-1 (the one tile i+2 is copied into)
   // Only the last key tile can be partial.  It is peeled off the loop so that the loop body has no masking
   // branch between S^T and the softmax, which lets the numerators of the first 32 keys be scheduled under
   // the MFMAs of the second 32.
@@ -441,7 +441,8 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
     __syncthreads();                                                                                    \
     const char* kbuf = lds[slot];                                                                       \
-    if (i + 2 < nt) dma(entry(i + 2), slot == 0 ? kRing - 1 : slot - 1);                                \
+    if (i + 2 < nt) dma(entry(i + 2), slot_prev);                                                       \
+    slot_prev = slot;                                                                                   \
     slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
     const int tile = entry(i);                                                                          \
     qk_tile<FP8, (WAVES > 8)>(w, kbuf, kbuf + kKBytes, lane);                                           \
