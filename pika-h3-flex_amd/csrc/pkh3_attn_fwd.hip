@@ -319,7 +319,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
   constexpr int kChunks = kTileBytes / 1024;  // 1 KiB pieces of a tile, dealt round-robin to the waves
   constexpr int kHalfBytes = kTileBytes / 2;  // K and V images of 32 keys
   // dense / phase 1: ring of kRing whole tiles; sparse phase 2: two stages of four row-private half tiles
-  constexpr int kLdsBytes = SPARSE && 8 * kHalfBytes > kRing * kTileBytes ? 8 * kHalfBytes : kRing * kTileBytes;
+  constexpr int kStageBytes = 32 * kD * 2;    // one wave's 32 x 128 bf16 output block, staged for the row-wise store
+  constexpr int kRingBytes = SPARSE && 8 * kHalfBytes > kRing * kTileBytes ? 8 * kHalfBytes : kRing * kTileBytes;
+  constexpr int kLdsBytes = kRingBytes > WAVES * kStageBytes ? kRingBytes : WAVES * kStageBytes;
   __shared__ __attribute__((aligned(1024))) char lds_raw[kLdsBytes];
   char(*lds)[kTileBytes] = (char(*)[kTileBytes])lds_raw;
   const int lane = threadIdx.x & 63;
@@ -510,13 +512,17 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
 #undef PKH3_HALF_LOOP
   }
 
-  // epilogue: O = O^T / l, bf16, 8-byte stores (4 consecutive d per register group)
+  // Epilogue: O = O^T / l in bf16.  A lane holds 4 consecutive d of one query per register group, which would
+  // make 8-byte stores scattered over 32 rows; instead each wave turns its 32 x 128 block around in its own
+  // 8 KiB of LDS (16-byte chunks XOR-swizzled by the row so both directions are conflict-free) and stores
+  // whole 256-byte rows, 16 bytes per lane.
   __bf16* ob = (__bf16*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
   const float lt = w.l + xhalf(w.l);
   const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-  const int q = q32 * 32 + (lane & 31);
-  if (q < p.Sq) {
-    __bf16* orow = ob + (int64_t)q * p.o_ss;
+  __syncthreads();  // every wave is done reading K/V tiles: the ring becomes staging space
+  char* stage = lds_raw + wave * kStageBytes;
+  {
+    const int qr = lane & 31;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -524,8 +530,17 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
         bf16x4 wv;
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) wv[rr] = (__bf16)(w.o[db][4 * g + rr] * inv);
-        *(bf16x4*)(orow + 32 * db + 8 * g + 4 * hh) = wv;
+        const int chunk = (4 * db + g) ^ (qr & 15);
+        *(bf16x4*)(stage + qr * 256 + chunk * 16 + 8 * hh) = wv;
       }
+  }
+  // same wave wrote and reads: the LDS counter orders the two, no barrier
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = 4 * i + (lane >> 4), c = lane & 15;
+    const bf16x8 v = *(const bf16x8*)(stage + row * 256 + ((c ^ (row & 15)) * 16));
+    const int q = q32 * 32 + row;
+    if (q < p.Sq) *(bf16x8*)(ob + (int64_t)q * p.o_ss + 8 * c) = v;
   }
 }
 
