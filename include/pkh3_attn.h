@@ -62,8 +62,12 @@ enum {
 
 /* flags */
 enum {
-  PKH3_FLAG_FP8_QK = 1u << 0 /* quantise normed+roped Q and K to fp8 e4m3 (OCP) with one absmax scale
-                                per (batch, head, 64-row block); P.V stays bf16 with fp32 accumulation */
+  PKH3_FLAG_FP8_QK = 1u << 0, /* quantise normed+roped Q and K to fp8 e4m3 (OCP) with one absmax scale
+                                 per (batch, head, 64-row block); P.V stays bf16 with fp32 accumulation */
+  PKH3_FLAG_LONG_KEY_KERNEL = 1u << 1 /* dense calls with at most 16 key tiles (Sk <= 1024) normally run a
+                                 short-key form of the kernel (small workgroups, three per CU); this flag
+                                 selects the long-key form for them too.  Same results to the tolerance of the
+                                 path; meant for tests and measurements */
 };
 
 typedef struct pkh3_attn_args {

@@ -24,6 +24,7 @@ PKH3_EARG = -9
 
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_HALF = 0, 1, 2
 FLAG_FP8_QK = 1
+FLAG_LONG_KEY_KERNEL = 2
 
 EXPORTS = (
     "pkh3_workspace_bytes",

@@ -46,7 +46,7 @@ int validate(const pkh3_attn_args* a, bool pointers) {
   if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Sk < 1) return fail(PKH3_ESHAPE, "B, H, Sq, Sk must be >= 1");
   if (a->B > 65535 || a->H > 65535) return fail(PKH3_ESHAPE, "B and H must be <= 65535");
   if (a->Sq > (1 << 24) || a->Sk > (1 << 24)) return fail(PKH3_ESHAPE, "Sq and Sk must be <= 2^24");
-  if (a->flags & ~(uint32_t)PKH3_FLAG_FP8_QK) return fail(PKH3_EARG, "unknown flag bits 0x%x", a->flags);
+  if (a->flags & ~(uint32_t)(PKH3_FLAG_FP8_QK | PKH3_FLAG_LONG_KEY_KERNEL)) return fail(PKH3_EARG, "unknown flag bits 0x%x", a->flags);
   if (a->rope_mode < PKH3_ROPE_NONE || a->rope_mode > PKH3_ROPE_HALF) return fail(PKH3_EARG, "bad rope_mode %d", a->rope_mode);
   if (!(a->softmax_scale == a->softmax_scale) || isinf(a->softmax_scale)) return fail(PKH3_EARG, "softmax_scale is not finite");
   if ((a->q_norm_w || a->k_norm_w) && !(a->norm_eps >= 0.f)) return fail(PKH3_EARG, "norm_eps must be >= 0");
@@ -143,7 +143,7 @@ void build(const pkh3_attn_args* a, Launch& L) {
   f.plan = a->blk_row_ptr ? (const int*)(ws + L.w.plan_off) : nullptr;
   f.plan_cnt = a->blk_row_ptr ? (const int*)(ws + L.w.plan_cnt_off) : nullptr;
   f.plan_stride = 5 * L.w.nKt;
-  f.kscale = k.scale_out; f.fp8 = fp8;
+  f.kscale = k.scale_out; f.fp8 = fp8; f.long_key_kernel = (a->flags & PKH3_FLAG_LONG_KEY_KERNEL) ? 1 : 0;
   f.kmax = (const float*)(ws + L.w.kmax_off);
 }
 

@@ -20,6 +20,9 @@
 // The transposed formulation keeps every per-query quantity (max, sum, rescale factor) a per-lane
 // scalar: no cross-lane traffic in the rescale, none between the two GEMMs.
 //
+// Short-key form (dense, at most 16 key tiles): 4 waves per workgroup, 32-key half tiles, three workgroups per
+// CU; see attn_fwd_kernel.
+//
 // Block-sparse variant.  A workgroup covers 4 query row-blocks (64 queries each, a wave pair per row-block).
 // Phase 1 walks the key tiles all four row-blocks keep, exactly like the dense kernel.  Phase 2 walks the
 // remaining tiles per row-block: every iteration gives each wave pair one 32-key half of a tile of its own
@@ -30,6 +33,8 @@
 namespace pkh3 {
 
 constexpr int kDenseWaves = 12;  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
+constexpr int kShortWaves = 4;   // short-key dense kernel: three 4-wave workgroups per CU
+constexpr int kShortMaxTiles = 16;  // key tiles up to which the short-key kernel is used
 constexpr int kSparseWaves = 8;  // the block-sparse kernel is built around 4 row-blocks x 2 waves (two per SIMD)
 constexpr int kRing = 3;               // LDS ring depth (tiles)
 constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
@@ -233,11 +238,21 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
 // ---- 32-key half tiles, used by the second phase of the block-sparse kernel -----------------------------
 // S^T (32 keys x 32 queries) into w.s[0]; kbuf/vbuf point at this half's K images (8 bf16 / 4 fp8 chunks)
 // and V images (8).
-template <bool FP8>
+// LEAN (three waves per SIMD): the K reads run 4 images ahead and only the fp8 path prefetches V (4 images).
+template <bool FP8, bool LEAN = false>
 __device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) w.s[0][i] = 0.f;
-  if constexpr (!FP8) {
+  if constexpr (!FP8 && LEAN) {
+    bf16x8 kf[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      w.s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], w.qf[i], w.s[0], 0, 0, 0);
+      if (i + 4 < 8) kf[i + 4] = *(const bf16x8*)(kbuf + ((i + 4) * 64 + lane) * 16);
+    }
+  } else if constexpr (!FP8) {
     bf16x8 kf[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
@@ -258,15 +273,19 @@ __device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, con
       const i32x8 b = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
       w.s[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, w.s[0], 0, 0, 0, 0, 0, 0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) w.vf[4 * ks + i] = *(const bf16x8*)(vbuf + ((4 * ks + i) * 64 + lane) * 16);
+      for (int i = 0; i < (LEAN ? 2 : 4); ++i) {
+        const int v = (LEAN ? 2 : 4) * ks + i;
+        w.vf[v] = *(const bf16x8*)(vbuf + (v * 64 + lane) * 16);
+      }
     }
   }
 }
 
 // Softmax numerators of w.s[0] and O^T += V^T P^T for one half tile (V images already in w.vf).
 // `lim` = keys of this half that exist (<= 0: none; only read when < 32).
-template <bool FP8, bool STATIC>
-__device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int lim, int lane) {
+// LEAN: the V images (beyond the 4 the fp8 path prefetched) are read here, 4 ahead of their MFMAs, from vbuf.
+template <bool FP8, bool STATIC, bool LEAN = false>
+__device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int lim, int lane, const char* vbuf = nullptr) {
   const int hh = lane >> 5;
   if (lim < 32) {
 #pragma unroll
@@ -307,20 +326,38 @@ __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int 
     pf[b2] = pk;
   }
   w.l = STATIC ? w.l + rsum : w.l * alpha + rsum;
+  if constexpr (LEAN) {
+    bf16x8 vg[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) w.o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w.vf[i], pf[i >> 2], w.o[i & 3], 0, 0, 0);
+    for (int i = 0; i < 4; ++i) vg[i] = FP8 ? w.vf[i] : *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      w.o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vg[i], pf[i >> 2], w.o[i & 3], 0, 0, 0);
+      if (i + 4 < 8) vg[i + 4] = *(const bf16x8*)(vbuf + ((i + 4) * 64 + lane) * 16);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w.o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w.vf[i], pf[i >> 2], w.o[i & 3], 0, 0, 0);
+  }
 }
 
+// WAVES == kShortWaves selects the short-key form of the dense kernel: 4 waves (one per SIMD, <= 168 VGPRs) and a
+// ring of 32-key half tiles in 48 KiB of LDS, so three workgroups share a CU and the Q load and O store of one
+// run under the tiles of the others.  With few key tiles that overlap is worth more than the three-fold K/V
+// copies cost (the K/V of such calls sit in L2).
 template <bool FP8, bool SPARSE, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void attn_fwd_kernel(FwdParams p) {
   static_assert(!SPARSE || WAVES == kSparseWaves, "block-sparse layout assumes 8 waves per workgroup");
+  constexpr bool SHORT = WAVES == kShortWaves;
+  static_assert(!(SHORT && SPARSE), "the short-key form is dense only");
   constexpr int kKBytes = FP8 ? kK8TileBytes : kKTileBytes;
   constexpr int kTileBytes = kKBytes + kVTileBytes;
   constexpr int kChunks = kTileBytes / 1024;  // 1 KiB pieces of a tile, dealt round-robin to the waves
   constexpr int kHalfBytes = kTileBytes / 2;  // K and V images of 32 keys
   // dense / phase 1: ring of kRing whole tiles; sparse phase 2: two stages of four row-private half tiles
   constexpr int kStageBytes = 32 * kD * 2;    // one wave's 32 x 128 bf16 output block, staged for the row-wise store
-  constexpr int kRingBytes = SPARSE && 8 * kHalfBytes > kRing * kTileBytes ? 8 * kHalfBytes : kRing * kTileBytes;
+  constexpr int kRingBytes = SHORT ? kRing * kHalfBytes
+                             : (SPARSE && 8 * kHalfBytes > kRing * kTileBytes ? 8 * kHalfBytes : kRing * kTileBytes);
   constexpr int kLdsBytes = kRingBytes > WAVES * kStageBytes ? kRingBytes : WAVES * kStageBytes;
   __shared__ __attribute__((aligned(1024))) char lds_raw[kLdsBytes];
   char(*lds)[kTileBytes] = (char(*)[kTileBytes])lds_raw;
@@ -358,8 +395,31 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
   };
   auto entry = [&](int i) { return SPARSE ? uniform_load(plan, i) : i; };  // i-th shared tile
 
+  // short-key form: halves of key tiles, [K half | V half] per ring slot; every wave copies the same share
+  constexpr int kKHalfB = kKBytes / 2, kVHalfB = kVTileBytes / 2;
+  const int n_half = (sk + 31) / 32;
+  auto dma_short = [&](int half, int slot) {
+    static_assert((kKHalfB / 1024) % kShortWaves == 0 && (kVHalfB / 1024) % kShortWaves == 0, "equal shares");
+    const char* g = p.kv + (int64_t)bh * p.kv_bh_stride + (int64_t)(half >> 1) * p.kv_tile_stride;
+    char* d = lds_raw + slot * kHalfBytes;
+    const int kb = half & 1;
+#pragma unroll
+    for (int i = 0; i < kKHalfB / 1024 / kShortWaves; ++i) {
+      const int ch = wave * (kKHalfB / 1024 / kShortWaves) + i;
+      lds_dma16(g + kb * kKHalfB + ch * 1024, lane_off, d + ch * 1024);
+    }
+#pragma unroll
+    for (int i = 0; i < kVHalfB / 1024 / kShortWaves; ++i) {
+      const int ch = wave * (kVHalfB / 1024 / kShortWaves) + i;
+      lds_dma16(g + kKBytes + kb * kVHalfB + ch * 1024, lane_off, d + kKHalfB + ch * 1024);
+    }
+  };
+
   WaveState<FP8> w;
-  if (nt > 0) {
+  if constexpr (SHORT) {
+    if (n_half > 0) dma_short(0, 0);
+    if (n_half > 1) dma_short(1, 1);
+  } else if (nt > 0) {
     dma(entry(0), 0);
     if (nt > 1) dma(entry(1), 1);
   }
@@ -447,11 +507,31 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
     slot_prev = slot;                                                                                   \
     slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
     const int tile = entry(i);                                                                          \
-    qk_tile<FP8, (WAVES > 8)>(w, kbuf, kbuf + kKBytes, lane);                                           \
+    qk_tile<FP8, (WAVES != kSparseWaves)>(w, kbuf, kbuf + kKBytes, lane);                                           \
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
-    softmax_pv_tile<FP8, STATIC, (WAVES > 8), MASKED>(w, kbuf + kKBytes, ct, tail, lane);                 \
+    softmax_pv_tile<FP8, STATIC, (WAVES != kSparseWaves), MASKED>(w, kbuf + kKBytes, ct, tail, lane);                 \
   }
-  if (static_max) {
+#define PKH3_SHORT_LOOP(STATIC)                                                                         \
+  for (int i = 0; i < n_half; ++i) {                                                                    \
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
+    __syncthreads();                                                                                    \
+    const char* hbuf = lds_raw + slot * kHalfBytes;                                                     \
+    if (i + 2 < n_half) dma_short(i + 2, slot_prev);                                                    \
+    slot_prev = slot;                                                                                   \
+    slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
+    qk_half<FP8, true>(w, hbuf, hbuf + kKHalfB, lane);                                                  \
+    const float ct = FP8 ? c * uniform_load(kscale, i >> 1) : c;                                        \
+    softmax_pv_half<FP8, STATIC, true>(w, ct, sk - 32 * i, lane, hbuf + kKHalfB);                       \
+  }
+  if constexpr (SHORT) {
+    if (static_max) {
+      PKH3_SHORT_LOOP(true)
+      PKH3_MFMA_DRAIN();
+    } else {
+      PKH3_SHORT_LOOP(false)
+      PKH3_MFMA_DRAIN();
+    }
+  } else if (static_max) {
     PKH3_TILE_LOOP(true, false, 0, nt - n_masked)
     PKH3_TILE_LOOP(true, true, nt - n_masked, nt)
     PKH3_MFMA_DRAIN();
@@ -461,6 +541,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void attn_fwd_kernel(FwdParams p) {
     PKH3_MFMA_DRAIN();
   }
 #undef PKH3_TILE_LOOP
+#undef PKH3_SHORT_LOOP
 
   if constexpr (SPARSE) {
     // Phase 2: the tiles that only some row-blocks keep.  Each row-block (a wave pair) walks its own list in
@@ -553,11 +634,14 @@ static void launch_variant(const FwdParams& p, hipStream_t st) {
 
 hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
   const bool sparse = p.plan != nullptr;
+  const bool short_keys = p.nKt <= kShortMaxTiles && !p.long_key_kernel;
   if (p.fp8) {
     if (sparse) launch_variant<true, true, kSparseWaves>(p, st);
+    else if (short_keys) launch_variant<true, false, kShortWaves>(p, st);
     else launch_variant<true, false, kDenseWaves>(p, st);
   } else {
     if (sparse) launch_variant<false, true, kSparseWaves>(p, st);
+    else if (short_keys) launch_variant<false, false, kShortWaves>(p, st);
     else launch_variant<false, false, kDenseWaves>(p, st);
   }
   return hipGetLastError();

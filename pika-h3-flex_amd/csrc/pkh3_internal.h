@@ -72,6 +72,7 @@ struct FwdParams {
   const float* kscale;      // [B*H, nKt] fp8 dequantisation scales of the K tiles
   const float* kmax;        // [B*H] largest K' row norm
   int fp8;
+  int long_key_kernel;  // never pick the short-key form
 };
 
 hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int* cnt, hipStream_t st);

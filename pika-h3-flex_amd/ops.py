@@ -62,7 +62,7 @@ def _f32(name: str, t: Optional[torch.Tensor], shape) -> Optional[torch.Tensor]:
 def fill_args(
     q, k, v, out, *, q_norm_weight=None, k_norm_weight=None, norm_eps=1e-6, rope_q=None, rope_k=None,
     rope_mode=_lib.ROPE_NONE, key_mask=None, block_mask: Optional[BlockMask] = None, fp8_qk=False,
-    softmax_scale: Optional[float] = None,
+    softmax_scale: Optional[float] = None, long_key_kernel: bool = False,
 ) -> Tuple[_lib.AttnArgs, list]:
     """Build ``pkh3_attn_args`` for these tensors.  Returns (args, keep_alive)."""
     for n, t in (("q", q), ("k", k), ("v", v), ("out", out)):
@@ -111,7 +111,7 @@ def fill_args(
             raise ValueError(f"block mask has {block_mask.row_ptr.numel() - 1} tile rows, need {nrow}")
         a.blk_row_ptr, a.blk_col_idx = block_mask.row_ptr.data_ptr(), block_mask.col_idx.data_ptr()
         keep += [block_mask.row_ptr, block_mask.col_idx]
-    a.flags = _lib.FLAG_FP8_QK if fp8_qk else 0
+    a.flags = (_lib.FLAG_FP8_QK if fp8_qk else 0) | (_lib.FLAG_LONG_KEY_KERNEL if long_key_kernel else 0)
     keep += [qw, kw]
     return a, keep
 

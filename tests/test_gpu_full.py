@@ -167,14 +167,15 @@ def test_golden_vectors():
             opts.update(block_mask=pk.BlockMask.from_dense(case["tile_map"], device="cuda"))
         if case.get("fp8"):
             opts.update(fp8_qk=True)
-        out = pk.attention(case["q"].cuda(), case["k"].cuda(), case["v"].cuda(), **opts)
-        torch.cuda.synchronize()
-        err, cos = O.max_abs_and_cosine(out.cpu(), case["out"])
-        print(f"golden {name}: max_abs={err:.3e} cos={cos:.7f}", flush=True)
-        if case.get("fp8"):
-            assert cos >= 0.995
-        else:
-            assert err <= 2e-2 and cos >= 0.9999
+        for long_form in (False, True):  # both forms of the dense kernel (the flag is ignored by the sparse one)
+            out = pk.attention(case["q"].cuda(), case["k"].cuda(), case["v"].cuda(), long_key_kernel=long_form, **opts)
+            torch.cuda.synchronize()
+            err, cos = O.max_abs_and_cosine(out.cpu(), case["out"])
+            print(f"golden {name} long_form={long_form}: max_abs={err:.3e} cos={cos:.7f}", flush=True)
+            if case.get("fp8"):
+                assert cos >= 0.995
+            else:
+                assert err <= 2e-2 and cos >= 0.9999
 
 
 class _Attn(torch.nn.Module):

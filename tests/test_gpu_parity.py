@@ -53,13 +53,17 @@ def _run_and_check(B, Sq, Sk, H, *, seed=0, norm=True, rope_mode=0, mask=None, s
         opts.update(rope_q=(f32(rope_q[0]), f32(rope_q[1])), rope_k=(f32(rope_k[0]), f32(rope_k[1])))
     if mask is not None:
         opts.update(key_mask=mask.to(dev))
-    out = pk.attention(q.to(dev), k.to(dev), v.to(dev), **opts)
-    torch.cuda.synchronize()
-    out = out.cpu()
-    assert torch.isfinite(out.float()).all()
-    err, cos = O.max_abs_and_cosine(out, ref)
-    print(f"B={B} Sq={Sq} Sk={Sk} H={H} rope={rope_mode} mask={mask is not None}: max_abs={err:.3e} cos={cos:.7f}", flush=True)
-    assert err <= max_abs and cos >= min_cos
+    # calls with at most 16 key tiles normally take the short-key form of the kernel: check the long-key form
+    # on the same inputs too, so both forms see every small case
+    for long_form in (True, False):
+        out = pk.attention(q.to(dev), k.to(dev), v.to(dev), long_key_kernel=long_form, **opts)
+        torch.cuda.synchronize()
+        out = out.cpu()
+        assert torch.isfinite(out.float()).all()
+        err, cos = O.max_abs_and_cosine(out, ref)
+        print(f"B={B} Sq={Sq} Sk={Sk} H={H} rope={rope_mode} mask={mask is not None} long_form={long_form}: "
+              f"max_abs={err:.3e} cos={cos:.7f}", flush=True)
+        assert err <= max_abs and cos >= min_cos
     return out, ref
 
 

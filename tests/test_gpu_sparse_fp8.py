@@ -75,8 +75,9 @@ def test_block_sparse_empty_rows_are_zero():
     assert torch.count_nonzero(out[:, 0:64]) > 0 and torch.count_nonzero(out[:, 128:192]) > 0
 
 
+@pytest.mark.parametrize("long_form", [False, True])
 @pytest.mark.parametrize("S,rope", [(256, 0), (1000, 1), (777, 2)])
-def test_fp8_qk(S, rope):
+def test_fp8_qk(S, rope, long_form):
     from oracle import attention_oracle as O
 
     q, k, v, gen = _inputs(1, S, S, 2, seed=100 + S)
@@ -89,7 +90,7 @@ def test_fp8_qk(S, rope):
         opts = dict(rope_q=tuple(t.float().contiguous().cuda() for t in tabs), rope_mode=rope)
     ref8 = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, fp8_qk=True, **ref_opts)
     ref = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, **ref_opts)
-    out = _call(q, k, v, q_norm_weight=_ones(), k_norm_weight=_ones(), fp8_qk=True, **opts)
+    out = _call(q, k, v, q_norm_weight=_ones(), k_norm_weight=_ones(), fp8_qk=True, long_key_kernel=long_form, **opts)
     err8, cos8 = O.max_abs_and_cosine(out, ref8)
     err, cos = O.max_abs_and_cosine(out, ref)
     print(f"fp8 S={S} rope={rope}: vs fp8 oracle max_abs={err8:.3e} cos={cos8:.6f}; vs unquantised max_abs={err:.3e} cos={cos:.6f}", flush=True)
