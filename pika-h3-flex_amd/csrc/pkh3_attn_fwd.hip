@@ -34,7 +34,11 @@ namespace pkh3 {
 
 constexpr int kDenseWaves = 12;  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
 constexpr int kShortWaves = 4;   // short-key dense kernel: three 4-wave workgroups per CU
+#ifdef PKH3_X_SHORTMAX
+constexpr int kShortMaxTiles = PKH3_X_SHORTMAX;
+#else
 constexpr int kShortMaxTiles = 16;  // key tiles up to which the short-key kernel is used
+#endif
 constexpr int kSparseWaves = 8;  // the block-sparse kernel is built around 4 row-blocks x 2 waves (two per SIMD)
 constexpr int kRing = 3;               // LDS ring depth (tiles)
 constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
@@ -284,10 +288,11 @@ __device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, con
 // Softmax numerators of w.s[0] and O^T += V^T P^T for one half tile (V images already in w.vf).
 // `lim` = keys of this half that exist (<= 0: none; only read when < 32).
 // LEAN: the V images (beyond the 4 the fp8 path prefetched) are read here, 4 ahead of their MFMAs, from vbuf.
-template <bool FP8, bool STATIC, bool LEAN = false>
+// FULL: the caller guarantees lim == 32, no masking code at all.
+template <bool FP8, bool STATIC, bool LEAN = false, bool FULL = false>
 __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int lim, int lane, const char* vbuf = nullptr) {
   const int hh = lane >> 5;
-  if (lim < 32) {
+  if (!FULL && lim < 32) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int key = 8 * (i / 4) + 4 * hh + (i % 4);
@@ -345,20 +350,29 @@ __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int 
 // ring of 32-key half tiles in 48 KiB of LDS, so three workgroups share a CU and the Q load and O store of one
 // run under the tiles of the others.  With few key tiles that overlap is worth more than the three-fold K/V
 // copies cost (the K/V of such calls sit in L2).
-template <bool FP8, bool SPARSE, int WAVES>
+// SPLIT (dense, 12 waves) is the form for the last, partly filled round of a long dense call: the workgroup takes
+// 128 queries instead of 384 and its three groups of 4 waves walk one third of the keys each (half tiles, a ring
+// per group), then add their partial results up through LDS.  Such a workgroup lasts a third as long, so the
+// CUs that would idle through a whole round of whole workgroups idle through a third of one.
+template <bool FP8, bool SPARSE, int WAVES, bool SPLIT = false>
 __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void attn_fwd_kernel(FwdParams p) {
   static_assert(!SPARSE || WAVES == kSparseWaves, "block-sparse layout assumes 8 waves per workgroup");
   constexpr bool SHORT = WAVES == kShortWaves;
-  static_assert(!(SHORT && SPARSE), "the short-key form is dense only");
+  constexpr bool HALFMODE = SHORT || SPLIT;             // rings of 32-key half tiles, 4 waves per ring
+  constexpr int GROUPS = SPLIT ? WAVES / kShortWaves : 1;  // key-range groups of the workgroup
+  static_assert(!(HALFMODE && SPARSE), "the half-tile forms are dense only");
+  static_assert(!SPLIT || WAVES % kShortWaves == 0, "whole groups of 4 waves");
   constexpr int kKBytes = FP8 ? kK8TileBytes : kKTileBytes;
   constexpr int kTileBytes = kKBytes + kVTileBytes;
   constexpr int kChunks = kTileBytes / 1024;  // 1 KiB pieces of a tile, dealt round-robin to the waves
   constexpr int kHalfBytes = kTileBytes / 2;  // K and V images of 32 keys
   // dense / phase 1: ring of kRing whole tiles; sparse phase 2: two stages of four row-private half tiles
   constexpr int kStageBytes = 32 * kD * 2;    // one wave's 32 x 128 bf16 output block, staged for the row-wise store
-  constexpr int kRingBytes = SHORT ? kRing * kHalfBytes
+  constexpr int kRingBytes = HALFMODE ? GROUPS * kRing * kHalfBytes
                              : (SPARSE && 8 * kHalfBytes > kRing * kTileBytes ? 8 * kHalfBytes : kRing * kTileBytes);
-  constexpr int kLdsBytes = kRingBytes > WAVES * kStageBytes ? kRingBytes : WAVES * kStageBytes;
+  constexpr int kMergeBytes = 64 * 64 * 4 + 2 * 64 * 4;  // SPLIT: one wave's O^T, row sums and row maxima in fp32
+  constexpr int kAfterBytes = SPLIT ? kShortWaves * kMergeBytes : WAVES * kStageBytes;  // LDS use after the loops
+  constexpr int kLdsBytes = kRingBytes > kAfterBytes ? kRingBytes : kAfterBytes;
   __shared__ __attribute__((aligned(1024))) char lds_raw[kLdsBytes];
   char(*lds)[kTileBytes] = (char(*)[kTileBytes])lds_raw;
   const int lane = threadIdx.x & 63;
@@ -367,14 +381,27 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
 
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD one contiguous run of
   // (batch, head, query tile) so the 32 CUs behind one L2 stream the same K/V at the same time.
-  const int nQt = (p.nQ64 * 2 + WAVES - 1) / WAVES;
-  const int total = p.B * p.H * nQt;
+  // A launch covers the units [p.unit0, p.unit0 + p.units); a unit is one workgroup's block of queries.
+  const int total = p.units;
   const int per_xcd = (total + 7) / 8;
   const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (lin >= total) return;
-  const int bh = lin / nQt, qt = lin % nQt;
+  const int unit = p.unit0 + lin;
+  const int group = SPLIT ? wave / kShortWaves : 0;       // which third of the keys (SPLIT)
+  const int wq = HALFMODE ? wave % kShortWaves : wave;    // which 32-query block of the unit
+  int bh, qt, q32;
+  if constexpr (SPLIT) {
+    // units are thirds of the 12-wave form's query tiles, so that a call can hand its last tiles to this form
+    const int nQt = (p.nQ64 * 2 + WAVES - 1) / WAVES;
+    bh = (unit / GROUPS) / nQt, qt = (unit / GROUPS) % nQt;
+    q32 = qt * WAVES + (unit % GROUPS) * kShortWaves + wq;
+  } else {
+    constexpr int kBlocks = HALFMODE ? kShortWaves : WAVES;  // 32-query blocks per unit
+    const int nQt = (p.nQ64 * 2 + kBlocks - 1) / kBlocks;
+    bh = unit / nQt, qt = unit % nQt;
+    q32 = qt * kBlocks + wq;
+  }
   const int b = bh / p.H, h = bh % p.H;
-  const int q32 = qt * WAVES + wave;  // 32-query block of this wave
 
   const int sk = p.row_cnt ? p.row_cnt[b] : p.Sk;
   const int nkt = (sk + kTileKeys - 1) / kTileKeys;
@@ -395,30 +422,34 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
   };
   auto entry = [&](int i) { return SPARSE ? uniform_load(plan, i) : i; };  // i-th shared tile
 
-  // short-key form: halves of key tiles, [K half | V half] per ring slot; every wave copies the same share
+  // half-tile forms: [K half | V half] per ring slot, one ring per group of 4 waves, every wave of the group
+  // copies the same share; group g walks the halves [h_begin, h_begin + n_mine)
   constexpr int kKHalfB = kKBytes / 2, kVHalfB = kVTileBytes / 2;
   const int n_half = (sk + 31) / 32;
+  const int h_begin = group * n_half / GROUPS;
+  const int n_mine = (group + 1) * n_half / GROUPS - h_begin;
+  char* ring = lds_raw + group * (kRing * kHalfBytes);
   auto dma_short = [&](int half, int slot) {
     static_assert((kKHalfB / 1024) % kShortWaves == 0 && (kVHalfB / 1024) % kShortWaves == 0, "equal shares");
     const char* g = p.kv + (int64_t)bh * p.kv_bh_stride + (int64_t)(half >> 1) * p.kv_tile_stride;
-    char* d = lds_raw + slot * kHalfBytes;
+    char* d = ring + slot * kHalfBytes;
     const int kb = half & 1;
 #pragma unroll
     for (int i = 0; i < kKHalfB / 1024 / kShortWaves; ++i) {
-      const int ch = wave * (kKHalfB / 1024 / kShortWaves) + i;
+      const int ch = wq * (kKHalfB / 1024 / kShortWaves) + i;
       lds_dma16(g + kb * kKHalfB + ch * 1024, lane_off, d + ch * 1024);
     }
 #pragma unroll
     for (int i = 0; i < kVHalfB / 1024 / kShortWaves; ++i) {
-      const int ch = wave * (kVHalfB / 1024 / kShortWaves) + i;
+      const int ch = wq * (kVHalfB / 1024 / kShortWaves) + i;
       lds_dma16(g + kKBytes + kb * kVHalfB + ch * 1024, lane_off, d + kKHalfB + ch * 1024);
     }
   };
 
   WaveState<FP8> w;
-  if constexpr (SHORT) {
-    if (n_half > 0) dma_short(0, 0);
-    if (n_half > 1) dma_short(1, 1);
+  if constexpr (HALFMODE) {
+    if (n_mine > 0) dma_short(h_begin, 0);
+    if (n_mine > 1) dma_short(h_begin + 1, 1);
   } else if (nt > 0) {
     dma(entry(0), 0);
     if (nt > 1) dma(entry(1), 1);
@@ -485,7 +516,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
   // small for the whole wave, exp2(logit) is a normal number in fp32 and in bf16 whatever the data, and so are
   // the row sums and O^T (at most 2^bound * keys * |v|), so no running max is needed at all.
   bool static_max = false;
-  if (nt > 0) {
+  if (HALFMODE ? n_half > 0 : nt > 0) {
     // margins: K' is rounded to bf16 (fp8: to e4m3, relative step 2^-4) after its norm was taken
     const float bound = sqrtf(qn2) * uniform_load(p.kmax, bh) * (FP8 ? p.c * 1.08f : 1.01f);
     static_max = __all(bound <= kStaticMaxLimit);
@@ -511,25 +542,77 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
     softmax_pv_tile<FP8, STATIC, (WAVES != kSparseWaves), MASKED>(w, kbuf + kKBytes, ct, tail, lane);                 \
   }
-#define PKH3_SHORT_LOOP(STATIC)                                                                         \
-  for (int i = 0; i < n_half; ++i) {                                                                    \
+  // Half-tile loop.  Every wave runs the same number of iterations (the longest group's), so the barriers match.
+  // A group's leading full halves take the copy of the code without masking; what is left -- at most the one
+  // partial half at the very end of the keys and one idle iteration of a shorter group -- takes the general copy.
+#define PKH3_SHORT_LOOP(STATIC, FULL, FROM, TO)                                                         \
+  for (int i = FROM; i < TO; ++i) {                                                                     \
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
     __syncthreads();                                                                                    \
-    const char* hbuf = lds_raw + slot * kHalfBytes;                                                     \
-    if (i + 2 < n_half) dma_short(i + 2, slot_prev);                                                    \
+    const char* hbuf = ring + slot * kHalfBytes;                                                        \
+    if (i + 2 < n_mine) dma_short(h_begin + i + 2, slot_prev);                                          \
     slot_prev = slot;                                                                                   \
     slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
-    qk_half<FP8, true>(w, hbuf, hbuf + kKHalfB, lane);                                                  \
-    const float ct = FP8 ? c * uniform_load(kscale, i >> 1) : c;                                        \
-    softmax_pv_half<FP8, STATIC, true>(w, ct, sk - 32 * i, lane, hbuf + kKHalfB);                       \
+    const int half = h_begin + i;                                                                       \
+    if (FULL || i < n_mine) {                                                                           \
+      qk_half<FP8, true>(w, hbuf, hbuf + kKHalfB, lane);                                                \
+      const float ct = FP8 ? c * uniform_load(kscale, half >> 1) : c;                                   \
+      softmax_pv_half<FP8, STATIC, true, FULL>(w, ct, sk - 32 * half, lane, hbuf + kKHalfB);            \
+    }                                                                                                   \
   }
-  if constexpr (SHORT) {
+  if constexpr (HALFMODE) {
+    const int n_iter = (n_half + GROUPS - 1) / GROUPS;
+    const int n_lead = max(0, min(n_mine, sk / 32 - h_begin));  // leading full halves of this group
     if (static_max) {
-      PKH3_SHORT_LOOP(true)
+      PKH3_SHORT_LOOP(true, true, 0, n_lead)
+      PKH3_SHORT_LOOP(true, false, n_lead, n_iter)
       PKH3_MFMA_DRAIN();
     } else {
-      PKH3_SHORT_LOOP(false)
+      PKH3_SHORT_LOOP(false, true, 0, n_lead)
+      PKH3_SHORT_LOOP(false, false, n_lead, n_iter)
       PKH3_MFMA_DRAIN();
+    }
+    if constexpr (SPLIT) {
+      // Add the groups' partial results into group 0, one group at a time through LDS.  On the bounded-logit
+      // path nothing was subtracted, so numerators and row sums just add; on the running-max path each side
+      // is first brought to the common maximum.
+      __syncthreads();  // every group is done with its ring
+      float* mbuf = (float*)(lds_raw + wq * kMergeBytes);
+#pragma unroll 1
+      for (int src = 1; src < GROUPS; ++src) {
+        if (group == src) {
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+              const f32x4 v4 = {w.o[db][4 * g4], w.o[db][4 * g4 + 1], w.o[db][4 * g4 + 2], w.o[db][4 * g4 + 3]};
+              *(f32x4*)(mbuf + ((db * 4 + g4) * 64 + lane) * 4) = v4;
+            }
+          mbuf[64 * 64 + lane] = w.l;
+          mbuf[64 * 64 + 64 + lane] = w.m;
+        }
+        __syncthreads();
+        if (group == 0) {
+          const float l2 = mbuf[64 * 64 + lane], m2 = mbuf[64 * 64 + 64 + lane];
+          float a1 = 1.0f, a2 = 1.0f;
+          if (!static_max) {
+            const float mn = fmaxf(w.m, m2);
+            a1 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w.m - mn);
+            a2 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m2 - mn);
+            w.m = mn;
+          }
+          w.l = w.l * a1 + l2 * a2;
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+              const f32x4 v4 = *(const f32x4*)(mbuf + ((db * 4 + g4) * 64 + lane) * 4);
+#pragma unroll
+              for (int rr = 0; rr < 4; ++rr) w.o[db][4 * g4 + rr] = w.o[db][4 * g4 + rr] * a1 + v4[rr] * a2;
+            }
+        }
+        __syncthreads();
+      }
     }
   } else if (static_max) {
     PKH3_TILE_LOOP(true, false, 0, nt - n_masked)
@@ -600,8 +683,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
   __bf16* ob = (__bf16*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
   const float lt = w.l + xhalf(w.l);
   const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-  __syncthreads();  // every wave is done reading K/V tiles: the ring becomes staging space
-  char* stage = lds_raw + wave * kStageBytes;
+  __syncthreads();  // every wave is done reading K/V tiles (SPLIT: and merge buffers): the LDS becomes staging space
+  if (SPLIT && group != 0) return;  // the merged result lives in group 0
+  char* stage = lds_raw + wq * kStageBytes;
   {
     const int qr = lane & 31;
 #pragma unroll
@@ -625,25 +709,48 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
   }
 }
 
-template <bool FP8, bool SPARSE, int WAVES>
-static void launch_variant(const FwdParams& p, hipStream_t st) {
-  const int nQt = (p.nQ64 * 2 + WAVES - 1) / WAVES;
-  const int total = p.B * p.H * nQt;
-  hipLaunchKernelGGL((attn_fwd_kernel<FP8, SPARSE, WAVES>), dim3((total + 7) / 8 * 8), dim3(64 * WAVES), 0, st, p);
+template <bool FP8, bool SPARSE, int WAVES, bool SPLIT = false>
+static void launch_variant(FwdParams p, int unit0, int units, hipStream_t st) {
+  p.unit0 = unit0;
+  p.units = units;
+  hipLaunchKernelGGL((attn_fwd_kernel<FP8, SPARSE, WAVES, SPLIT>), dim3((units + 7) / 8 * 8), dim3(64 * WAVES), 0, st, p);
+}
+
+template <bool FP8>
+static void launch_fp(const FwdParams& p, int cus, hipStream_t st) {
+  const int nQ32 = p.nQ64 * 2;
+  auto units = [&](int blocks) { return p.B * p.H * ((nQ32 + blocks - 1) / blocks); };
+  if (p.plan) return launch_variant<FP8, true, kSparseWaves>(p, 0, units(kSparseWaves), st);
+  if (p.nKt <= kShortMaxTiles && !p.long_key_kernel) return launch_variant<FP8, false, kShortWaves>(p, 0, units(kShortWaves), st);
+  // Long dense call: one workgroup per CU at a time, so the call runs in rounds of `cus` workgroups.  When the
+  // last round would be less than two thirds full, its query tiles go to the SPLIT form instead (three
+  // workgroups of a third of the duration each per tile), launched behind the whole rounds.
+  const int n = units(kDenseWaves);
+  const int whole = cus > 0 ? n / cus * cus : n, rest = n - whole;
+  constexpr int kGroups = kDenseWaves / kShortWaves;
+  if (whole > 0 && rest > 0 && rest * kGroups <= 2 * cus && !p.long_key_kernel) {
+    launch_variant<FP8, false, kDenseWaves>(p, 0, whole, st);
+    launch_variant<FP8, false, kDenseWaves, true>(p, whole * kGroups, rest * kGroups, st);
+  } else {
+    launch_variant<FP8, false, kDenseWaves>(p, 0, n, st);
+  }
 }
 
 hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
-  const bool sparse = p.plan != nullptr;
-  const bool short_keys = p.nKt <= kShortMaxTiles && !p.long_key_kernel;
-  if (p.fp8) {
-    if (sparse) launch_variant<true, true, kSparseWaves>(p, st);
-    else if (short_keys) launch_variant<true, false, kShortWaves>(p, st);
-    else launch_variant<true, false, kDenseWaves>(p, st);
-  } else {
-    if (sparse) launch_variant<false, true, kSparseWaves>(p, st);
-    else if (short_keys) launch_variant<false, false, kShortWaves>(p, st);
-    else launch_variant<false, false, kDenseWaves>(p, st);
+  // CUs of the current device, asked once per device
+  static int cu_count[64] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev >= 0 && dev < 64 && cu_count[dev] == 0) {
+    int n = 0;
+    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    cu_count[dev] = n;
   }
+  const int cus = dev >= 0 && dev < 64 ? cu_count[dev] : 0;
+  if (p.fp8) launch_fp<true>(p, cus, st);
+  else launch_fp<false>(p, cus, st);
   return hipGetLastError();
 }
 

@@ -72,7 +72,8 @@ struct FwdParams {
   const float* kscale;      // [B*H, nKt] fp8 dequantisation scales of the K tiles
   const float* kmax;        // [B*H] largest K' row norm
   int fp8;
-  int long_key_kernel;  // never pick the short-key form
+  int long_key_kernel;  // only the plain long-key form (no short-key form, no split last round)
+  int unit0, units;     // filled per launch: the workgroup units [unit0, unit0 + units) this launch covers
 };
 
 hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int* cnt, hipStream_t st);
