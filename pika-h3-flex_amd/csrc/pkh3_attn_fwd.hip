@@ -34,11 +34,7 @@ namespace pkh3 {
 
 constexpr int kDenseWaves = 12;  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
 constexpr int kShortWaves = 4;   // short-key dense kernel: three 4-wave workgroups per CU
-#ifdef PKH3_X_SHORTMAX
-constexpr int kShortMaxTiles = PKH3_X_SHORTMAX;
-#else
 constexpr int kShortMaxTiles = 16;  // key tiles up to which the short-key kernel is used
-#endif
 constexpr int kSparseWaves = 8;  // the block-sparse kernel is built around 4 row-blocks x 2 waves (two per SIMD)
 constexpr int kRing = 3;               // LDS ring depth (tiles)
 constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
