@@ -11,17 +11,22 @@
 //
 // Math per tile, all on the 32x32 MFMA shapes (see pkh3_common.h for the operand images):
 //   S^T = K' Q'^T      A = K image (LDS), B = Q image (VGPR)      -> lane l holds query l%32, 16 keys / block
-//                      (bf16: 16 x 32x32x16; fp8: 4 x 32x32x64 on e4m3 images, S^T rescaled by the
-//                      per-64-row-block dequantisation scales inside the softmax multiply)
-//   online softmax     row max: in-lane over the keys + one exchange with lane l^32; exp2 with the
-//                      softmax scale folded in; row sum kept per half-wave and merged once at the end;
-//                      the running max is only raised when exceeded by 2^8, so the O^T rescale is rare
+//                      (bf16: 16 x 32x32x16, Q' carries softmax_scale * log2(e) so S^T is in the log2 domain;
+//                      fp8: 4 x 32x32x64 on e4m3 images, S^T rescaled by the per-64-row-block dequantisation
+//                      scales in the softmax multiply)
+//   softmax            bounded-logit path (the usual one): |q_i| * max_j |k_j| bounds every logit of the wave's
+//                      queries; when that bound is small, exp2(logit) needs no maximum at all.  Otherwise the
+//                      online form: row max in-lane over the keys + one exchange with lane l^32, raised only
+//                      when exceeded by 2^8 so the O^T rescale is rare.  Row sum kept per half-wave, merged once
+//                      at the end.
 //   O^T += V^T P^T     A = V image (LDS), B = P packed to bf16 straight from the S^T registers
 // The transposed formulation keeps every per-query quantity (max, sum, rescale factor) a per-lane
-// scalar: no cross-lane traffic in the rescale, none between the two GEMMs.
+// scalar: no cross-lane traffic in the rescale, none between the two GEMMs.  O leaves through LDS, turned
+// around into whole 256-byte rows.
 //
-// Short-key form (dense, at most 16 key tiles): 4 waves per workgroup, 32-key half tiles, three workgroups per
-// CU; see attn_fwd_kernel.
+// Other forms of the dense kernel (see attn_fwd_kernel): the short-key form (at most 16 key tiles: 4 waves per
+// workgroup, 32-key half tiles, three workgroups per CU) and the split form for a thinly filled last round of
+// a long call (128 queries per workgroup, its three groups of 4 waves walk a third of the keys each).
 //
 // Block-sparse variant.  A workgroup covers 4 query row-blocks (64 queries each, a wave pair per row-block).
 // Phase 1 walks the key tiles all four row-blocks keep, exactly like the dense kernel.  Phase 2 walks the
