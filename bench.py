@@ -128,6 +128,8 @@ def main() -> int:
             roofline["mfma_probe"] = cases
             if cases.get("random"):
                 roofline["frac_of_measured_random_operand_ceiling"] = round(achieved / cases["random"]["tflops"], 4)
+            if cases.get("lds"):
+                roofline["frac_of_lds_fed_mfma_stream"] = round(achieved / cases["lds"]["tflops"], 4)
             if cases.get("attention"):
                 roofline["frac_of_attention_shaped_ceiling"] = round(achieved / cases["attention"]["tflops"], 4)
         except Exception as exc:  # the probe is informational only

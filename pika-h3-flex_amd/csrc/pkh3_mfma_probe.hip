@@ -4,6 +4,8 @@
 //
 //   "ones"      dependency-free MFMA stream, all-ones operands, 8 waves per CU, no memory traffic
 //   "random"    the same stream with random operands: every bit toggles, the part is power-limited and clocks lower
+//   "lds"       the random-operand stream with the A operand of every MFMA read from LDS (one 1 KiB image per MFMA,
+//               as the attention kernels do), 12 waves per CU, still no other instructions and no HBM traffic
 //   "attention" 12 waves per CU walking an attention-shaped tile loop with no HBM traffic at all: 16 MFMAs whose A
 //               operands are 1 KiB LDS images (two accumulate chains of 8, like S^T = K Q^T), 32 exp2 + 16 packed
 //               bf16 conversions + 16 dot2 row sums, 16 more MFMAs with LDS A operands and the converted values
@@ -12,7 +14,8 @@
 // The published 2.5 PFLOP/s bf16 dense figure corresponds to every MFMA issue slot used at the boost clock.  The
 // probe prints, for each case, the achieved rate, the average core clock over the run (core-clock counter against
 // the 100 MHz wall-clock counter) and the share of MFMA issue slots used at that clock ("pipe").  "random" is the
-// ceiling of any bf16 MFMA kernel with real data on the box; "attention" is the ceiling of this kernel structure
+// ceiling of any bf16 MFMA kernel with real data on the box; "lds" is what is left of it when the operands come
+// through LDS (the reads cost power, the clock drops further); "attention" is the ceiling of this kernel structure
 // before K/V streaming, Q/O traffic and softmax bookkeeping are added.
 //
 // Usage: pkh3_mfma_probe [iterations]     prints one JSON line per case.
@@ -72,6 +75,41 @@ __global__ __launch_bounds__(512) void mfma_stream(float* out, int iters, Clocks
 }
 
 constexpr int kAttnWaves = 12;
+
+__global__ __launch_bounds__(64 * kAttnWaves, 1) void lds_fed_stream(float* out, int iters, Clocks* clk) {
+  __shared__ __attribute__((aligned(1024))) char lds[32768];
+  const int lane = threadIdx.x & 63;
+  bf16x8 b[8];
+  for (int n = 0; n < 8; ++n) b[n] = random_image(threadIdx.x * 31u + n);
+  for (int i = threadIdx.x; i < 32768 / 16; i += 64 * kAttnWaves) ((bf16x8*)lds)[i] = random_image(i * 7u + 3u);
+  __syncthreads();
+  f32x16 acc[4];
+  for (int n = 0; n < 4; ++n)
+    for (int i = 0; i < 16; ++i) acc[n][i] = 0.f;
+  const long long c0 = clock64(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+    asm volatile("" ::: "memory");  // the images are read again every iteration
+    bf16x8 a[32];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[i] = *(const bf16x8*)(lds + (i * 64 + lane) * 16);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[i & 7], acc[i & 3], 0, 0, 0);
+      if (i + 4 < 32) a[i + 4] = *(const bf16x8*)(lds + ((i + 4) * 64 + lane) * 16);
+    }
+    if ((it & 63) == 63) {
+#pragma unroll
+      for (int n = 0; n < 4; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[n][i] *= 1e-6f;
+    }
+  }
+  stamp(clk, c0, w0);
+  float s = 0.f;
+  for (int n = 0; n < 4; ++n)
+    for (int i = 0; i < 16; ++i) s += acc[n][i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
 
 __global__ __launch_bounds__(64 * kAttnWaves, 1) void attention_shaped(float* out, int iters, Clocks* clk) {
   __shared__ __attribute__((aligned(1024))) char lds[32768];  // 16 "K" images, then 16 "V" images
@@ -159,14 +197,15 @@ int main(int argc, char** argv) {
   hipEvent_t e0, e1;
   CK(hipEventCreate(&e0));
   CK(hipEventCreate(&e1));
-  const char* names[3] = {"ones", "random", "attention"};
-  for (int mode = 0; mode < 3; ++mode) {
-    const int waves = mode == 2 ? kAttnWaves : 8;
+  const char* names[4] = {"ones", "random", "lds", "attention"};
+  for (int mode = 0; mode < 4; ++mode) {
+    const int waves = mode >= 2 ? kAttnWaves : 8;
     float ms = 0.f;
     for (int rep = 0; rep < 2; ++rep) {  // first repetition warms up
       CK(hipEventRecord(e0));
       if (mode == 0) hipLaunchKernelGGL(mfma_stream<false>, dim3(cus), dim3(512), 0, 0, out, iters, clk);
       else if (mode == 1) hipLaunchKernelGGL(mfma_stream<true>, dim3(cus), dim3(512), 0, 0, out, iters, clk);
+      else if (mode == 2) hipLaunchKernelGGL(lds_fed_stream, dim3(cus), dim3(64 * kAttnWaves), 0, 0, out, iters, clk);
       else hipLaunchKernelGGL(attention_shaped, dim3(cus), dim3(64 * kAttnWaves), 0, 0, out, iters, clk);
       CK(hipGetLastError());
       CK(hipEventRecord(e1));
