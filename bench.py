@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per attention-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00,
 # factors from a 1 GiB copy); figures and commands in profiles/attn_fwd_kernel_480p_bf16.md and
 # profiles/attn_fwd_kernel_480p_sparse_fp8.md
-MEASURED_TRAFFIC_BYTES = {"480p": 3.96e9, "480p-sparse-fp8": 2.11e10}
+MEASURED_TRAFFIC_BYTES = {"480p": 3.96e9, "480p-sparse-fp8": 2.12e10}
 
 
 def main() -> int:
