@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define PKH3_VERSION 100
+#define PKH3_VERSION 101
 
 enum {
   PKH3_OK = 0,
