@@ -36,7 +36,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="480p", choices=["plumbing", "480p", "768p", "joint", "cross", "480p-sparse", "480p-sparse-fp8", "480p-fp8"])
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--cpu-rows", type=int, default=16384, help="query rows of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-rows", type=int, default=32768, help="query rows of the CPU baseline sample (0 = skip)")
     ap.add_argument("--kernel-iters", type=int, default=10)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy, a kernel of known traffic for scaling profiler byte counters")
