@@ -96,11 +96,17 @@ def main() -> int:
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # the K timed steps, bracketed by synchronisation; per-step events (same stream) give median and minimum
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         step()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    ms_median, ms_min = per_step[len(per_step) // 2], per_step[0]
     value = flops / (ms_per_step * 1e-3) / 1e12
 
     kernel_ms = pk.time_attention_kernel(inp.q, inp.k, inp.v, iters=args.kernel_iters, **opts)
@@ -159,7 +165,8 @@ def main() -> int:
         "dtype": "fp8-e4m3 QK^T + bf16 PV" if fp8 else "bf16", "data": "synthetic",
         "config": {"workload": f"{args.workload} attention layer: B={B}, H={H}, D={D}, Sq={Sq}, Sk={Sk}, "
                                f"QK-RMSNorm + 3-axis RoPE, non-causal" + (f", block-sparse density {density:.3f}" if density < 1 else ""),
-                   "seed": args.seed, "pct_of_mfma_peak": round(100.0 * value / peak, 2)},
+                   "seed": args.seed, "pct_of_mfma_peak": round(100.0 * value / peak, 2),
+                   "ms_per_step_median": round(ms_median, 4), "ms_per_step_min": round(ms_min, 4)},
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
