@@ -186,7 +186,7 @@ def test_bound_path_and_running_max_path_agree():
     assert not torch.equal(out_small, out_big)
 
 
-@pytest.mark.parametrize("variant", ["dense_rope_mask", "sparse_fp8"])
+@pytest.mark.parametrize("variant", ["dense_rope_mask", "sparse_fp8", "long_dense_split_last_round"])
 def test_hip_graph_replays_match_eager(variant):
     """The layer call allocates nothing and only launches kernels on the caller's stream, so it can be captured
     into a HIP graph.  Every replay, with fresh inputs in the captured buffers and eager work in between, must
@@ -194,6 +194,8 @@ def test_hip_graph_replays_match_eager(variant):
     import pika_h3_flex_amd as pk
 
     B, S, H, D = 1, 333, 2, 128
+    if variant == "long_dense_split_last_round":
+        S, H = 4200, 24  # 264 query tiles on a 256-CU part: two launches (whole rounds, then the split form)
     gen = torch.Generator().manual_seed(91)
     dev = "cuda"
     q, k, v = (_rand((B, S, H, D), gen).to(dev) for _ in range(3))
@@ -204,12 +206,14 @@ def test_hip_graph_replays_match_eager(variant):
         cos, sin = pk.rope_tables(pos.to(dev))
         mask = (torch.rand((B, S), generator=gen) < 0.7).to(dev)
         opts.update(rope_mode=1, rope_q=(cos, sin), key_mask=mask)
+    elif variant == "long_dense_split_last_round":
+        pass
     else:
         tm = torch.rand((6, 6), generator=gen) < 0.5
         tm |= torch.eye(6, dtype=torch.bool)
         opts.update(block_mask=pk.BlockMask.from_dense(tm, device=dev), fp8_qk=True)
     out = torch.empty_like(q)
-    ws = torch.empty(1 << 22, dtype=torch.uint8, device=dev)
+    ws = torch.empty(1 << 27, dtype=torch.uint8, device=dev)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
