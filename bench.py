@@ -48,6 +48,9 @@ def main() -> int:
 
     import torch
 
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()  # loads what is built; compiles only when there is nothing
     import pika_h3_flex_amd as pk
     from pika_h3_flex_amd import workloads
 

@@ -10,6 +10,10 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # use the library that is built; compile it only when there is none
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()
 
 
 @pytest.fixture(scope="session")
