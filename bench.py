@@ -24,9 +24,31 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}  # MI355X dense MFMA, published
 HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per attention-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00,
-# factors from a 1 GiB copy); figures and commands in profiles/attn_fwd_kernel_480p_bf16.md and
-# profiles/attn_fwd_kernel_480p_sparse_fp8.md
-MEASURED_TRAFFIC_BYTES = {"480p": 3.96e9, "480p-sparse-fp8": 2.12e10}
+# factors from a 1 GiB copy) in earlier profiling runs of the same command, not in this run: (bytes, file that holds
+# the counter values and the commands)
+MEASURED_TRAFFIC = {
+    "480p": (3.96e9, "profiles/attn_fwd_kernel_480p_bf16.md"),
+    "480p-sparse-fp8": (2.12e10, "profiles/attn_fwd_kernel_480p_sparse_fp8.md"),
+}
+
+
+def host_cpu():
+    """(model name, physical cores) of the host from /proc/cpuinfo; physical = distinct (package, core id) pairs."""
+    model, cores = "unknown", set()
+    try:
+        phys = "0"
+        for line in open("/proc/cpuinfo"):
+            key, _, val = line.partition(":")
+            key, val = key.strip(), val.strip()
+            if key == "model name":
+                model = val
+            elif key == "physical id":
+                phys = val
+            elif key == "core id":
+                cores.add((phys, val))
+    except OSError:
+        pass
+    return model, (len(cores) or os.cpu_count() or 0)
 
 
 def main() -> int:
@@ -116,33 +138,9 @@ def main() -> int:
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS["fp8" if fp8 else "bf16"]
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "attn_fwd_kernel",
+                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
+                "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1], "kernel": "attn_fwd_kernel",
                 "kernel_ms": round(kernel_ms, 4), "flops_per_launch": flops}
-
-    # calibration: what this box sustains on bf16 MFMA work with nothing else in the way -- a pure MFMA stream with
-    # all-ones and with random operands (the part is power-limited on real data), and an attention-shaped tile
-    # loop fed from LDS with no HBM traffic (see pika-h3-flex_amd/csrc/pkh3_mfma_probe.hip)
-    probe = os.path.join(ROOT, "pika-h3-flex_amd", "pkh3_mfma_probe")
-    if os.path.exists(probe) and not fp8:
-        import subprocess
-
-        try:
-            res = subprocess.run([probe, "20000"], capture_output=True, text=True, timeout=120)
-            cases = {}
-            for line in res.stdout.splitlines():
-                if line.startswith("{"):
-                    d = json.loads(line)
-                    cases[d["operands"]] = {"tflops": d["tflops"], "core_clock_ghz": d["core_clock_ghz"],
-                                            "mfma_pipe_busy": d["mfma_pipe_busy"]}
-            roofline["mfma_probe"] = cases
-            if cases.get("random"):
-                roofline["frac_of_measured_random_operand_ceiling"] = round(achieved / cases["random"]["tflops"], 4)
-            if cases.get("lds"):
-                roofline["frac_of_lds_fed_mfma_stream"] = round(achieved / cases["lds"]["tflops"], 4)
-            if cases.get("attention"):
-                roofline["frac_of_attention_shaped_ceiling"] = round(achieved / cases["attention"]["tflops"], 4)
-        except Exception as exc:  # the probe is informational only
-            roofline["mfma_probe"] = f"probe failed: {exc}"
 
     cpu = None
     if args.cpu_rows > 0:
@@ -157,7 +155,9 @@ def main() -> int:
         secs, threads = cpu_sdpa.time_cpu_baseline(inp.q, inp.k, inp.v, sample_rows=rows, **cpu_opts)
         sk_eff = Sk if inp.key_mask is None else int(inp.key_mask.sum())
         cpu_flops = 4.0 * rows * sk_eff * D * H
+        cpu_model, cpu_physical = host_cpu()
         cpu = {"value": round(cpu_flops / secs / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+               "cpu_model": cpu_model, "physical_cores": cpu_physical,
                "sample": f"torch CPU F.scaled_dot_product_attention fp32 (+RMSNorm, RoPE in torch) on the first {rows} of {Sq} "
                          f"query rows x all {Sk} keys x {H} heads, dense, one call of {secs:.2f} s; rate scales linearly in rows"}
 

@@ -23,7 +23,8 @@
  * Conventions
  *   - plain pointers and sizes only; every buffer is owned by the caller and lives in device
  *     memory (HBM) unless stated; the library allocates nothing.
- *   - all work is enqueued on `stream` (a hipStream_t passed as void*); no call synchronises.
+ *   - all work is enqueued on `stream` (a hipStream_t passed as void*); no call declared in this header
+ *     synchronises (the benchmark hook in pkh3_attn_bench.h does, and is kept apart for that reason).
  *   - strides are in ELEMENTS; the innermost (head-dim) stride is 1 and D must be 128.
  *   - return value 0 = success, negative = PKH3_E* below.  Arguments are validated on the host
  *     before any HIP call, so argument errors are reported without a GPU.
@@ -125,11 +126,6 @@ int pkh3_version(void);
 const char* pkh3_strerror(int code);
 /* Message of the last failing call on this thread ("" if none). */
 const char* pkh3_last_error(void);
-
-/* Timing hook for benchmarks: runs `iters` back-to-back launches of ONLY the attention kernel of the
-   given call (the prologue that normalises/rotates/lays out K,V and Q runs once before), brackets them
-   with HIP events on `stream`, and returns the mean milliseconds per launch in *ms_out.  Synchronises. */
-int pkh3_attn_time_kernel(const pkh3_attn_args* a, void* stream, int iters, float* ms_out);
 
 #ifdef __cplusplus
 }

@@ -55,7 +55,7 @@ def rms_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> tor
     x = x.to(torch.float64)
     y = x * torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps)
     if weight is not None:
-        y = y * weight.to(torch.float64)
+        y = y * weight.to(device=x.device, dtype=torch.float64)
     return y
 
 
@@ -71,7 +71,7 @@ def rope_tables(position_ids: torch.Tensor, axes_dims=(32, 48, 48), theta: float
             raise ValueError("axis dims must be even")
         i = torch.arange(n // 2, dtype=torch.float64)
         freq = torch.pow(torch.tensor(float(theta), dtype=torch.float64), -2.0 * i / n)
-        cols.append(pos[:, a : a + 1] * freq[None, :])
+        cols.append(pos[:, a : a + 1] * freq.to(pos.device)[None, :])
     ang = torch.cat(cols, dim=1)
     return torch.cos(ang), torch.sin(ang)
 
@@ -81,8 +81,8 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, mode: int)
     if mode == ROPE_NONE:
         return x
     x = x.to(torch.float64)
-    c = cos.to(torch.float64)[None, :, None, :]
-    s = sin.to(torch.float64)[None, :, None, :]
+    c = cos.to(device=x.device, dtype=torch.float64)[None, :, None, :]
+    s = sin.to(device=x.device, dtype=torch.float64)[None, :, None, :]
     if mode == ROPE_INTERLEAVED:
         x0, x1 = x[..., 0::2], x[..., 1::2]
         y = torch.empty_like(x)
@@ -111,25 +111,34 @@ def fp8_e4m3_round(x: np.ndarray) -> np.ndarray:
     return np.sign(x) * q
 
 
+def fp8_e4m3_round_torch(x: torch.Tensor) -> torch.Tensor:
+    """The same rounding through torch's ``float8_e4m3fn`` cast (float32 in, float64 out), usable on
+    any device.  Pinned against :func:`fp8_e4m3_round` in tests/test_oracle.py; inputs must lie in
+    [-448, 448] (the cast does not saturate), which the absmax scaling below guarantees."""
+    return x.to(torch.float32).to(torch.float8_e4m3fn).to(torch.float64)
+
+
 def fake_quant_fp8_blocks(x: torch.Tensor, block: int = TILE) -> Tuple[torch.Tensor, torch.Tensor]:
     """Quantise ``x [B, S, H, D]`` to e4m3 with one absmax scale per (batch, head, ``block`` rows)
     and return (dequantised float64 tensor, scales ``[B, H, ceil(S/block)]``).  The scale and the
-    division follow float32 arithmetic (scale = absmax / 448, value * (1 / scale))."""
+    division follow float32 arithmetic (scale = absmax / 448, value * (1 / scale)).  Runs on the
+    device ``x`` lives on: NumPy rounding on the host, torch's e4m3 cast elsewhere."""
     B, S, H, D = x.shape
     nb = (S + block - 1) // block
-    x32 = x.to(torch.float32)
-    out = torch.zeros((B, S, H, D), dtype=torch.float64)
-    scales = torch.ones((B, H, nb), dtype=torch.float32)
-    for i in range(nb):
-        blk = x32[:, i * block : (i + 1) * block]                  # [B, r, H, D]
-        amax = blk.abs().amax(dim=(1, 3))                           # [B, H]
-        sc = torch.where(amax > 0, amax * np.float32(1.0 / FP8_MAX), torch.ones_like(amax))
-        inv = (torch.ones_like(sc) / sc)[:, None, :, None]
-        scaled = (blk * inv).to(torch.float64).numpy()
-        deq = torch.from_numpy(fp8_e4m3_round(scaled)) * sc.to(torch.float64)[:, None, :, None]
-        out[:, i * block : (i + 1) * block] = deq
-        scales[:, :, i] = sc
-    return out, scales
+    dev = x.device
+    x32 = torch.zeros((B, nb * block, H, D), dtype=torch.float32, device=dev)
+    x32[:, :S] = x.to(torch.float32)
+    blk = x32.view(B, nb, block, H, D)
+    amax = blk.abs().amax(dim=(2, 4))                                   # [B, nb, H]
+    sc = torch.where(amax > 0, amax * np.float32(1.0 / FP8_MAX), torch.ones_like(amax))
+    inv = (torch.ones_like(sc) / sc)[:, :, None, :, None]
+    scaled = blk * inv                                                  # float32, |.| <= 448
+    if dev.type == "cpu":
+        q = torch.from_numpy(fp8_e4m3_round(scaled.to(torch.float64).numpy()))
+    else:
+        q = fp8_e4m3_round_torch(scaled)
+    deq = (q * sc.to(torch.float64)[:, :, None, :, None]).view(B, nb * block, H, D)[:, :S]
+    return deq.contiguous(), sc.permute(0, 2, 1).contiguous()
 
 
 # ---------------------------------------------------------------------------------------------
@@ -147,31 +156,35 @@ def attention(
     key_mask: Optional[torch.Tensor] = None, tile_map: Optional[torch.Tensor] = None,
     q_rows: Optional[torch.Tensor] = None, chunk: int = 1024,
 ) -> torch.Tensor:
-    """Explicit float64 attention over ``[B, S, H, D]`` tensors.
+    """Explicit float64 attention over ``[B, S, H, D]`` tensors, on the device they live on.
 
     ``key_mask`` bool ``[B, Sk]`` (True = attend); ``tile_map`` bool 64x64-tile map.  A query row with
     no key left gets zeros.  ``q_rows`` (1-D long) restricts the computation to those query rows
     (the result then has ``len(q_rows)`` rows); the tile row of query r is ``r // 64``.
     """
     q, k, v = q.to(torch.float64), k.to(torch.float64), v.to(torch.float64)
+    dev = q.device
     B, Sq, H, D = q.shape
     Sk = k.shape[1]
     sc = 1.0 / math.sqrt(D) if scale is None else float(scale)
-    rows = torch.arange(Sq) if q_rows is None else q_rows.to(torch.long)
-    out = torch.zeros((B, rows.numel(), H, D), dtype=torch.float64)
+    rows = torch.arange(Sq, device=dev) if q_rows is None else q_rows.to(device=dev, dtype=torch.long)
+    out = torch.zeros((B, rows.numel(), H, D), dtype=torch.float64, device=dev)
     kt = k.permute(0, 2, 3, 1)  # [B, H, D, Sk]
     vt = v.permute(0, 2, 1, 3)  # [B, H, Sk, D]
+    km = None if key_mask is None else key_mask.to(device=dev, dtype=torch.bool)[:, None, None, :]
+    tmap = None if tile_map is None else tile_map.to(device=dev, dtype=torch.bool)
     for c0 in range(0, rows.numel(), chunk):
         r = rows[c0 : c0 + chunk]
         qc = q[:, r].permute(0, 2, 1, 3)  # [B, H, r, D]
         s = torch.matmul(qc, kt) * sc     # [B, H, r, Sk]
-        allow = torch.ones((B, 1, r.numel(), Sk), dtype=torch.bool)
-        if key_mask is not None:
-            allow = allow & key_mask.to(torch.bool)[:, None, None, :]
-        if tile_map is not None:
-            tm = tile_map.to(torch.bool)[r // TILE]                      # [r, nKt]
-            allow = allow & tm.repeat_interleave(TILE, 1)[:, :Sk][None, None]
-        s = s.masked_fill(~allow, float("-inf"))
+        allow = None
+        if km is not None:
+            allow = km
+        if tmap is not None:
+            tm = tmap[r // TILE].repeat_interleave(TILE, 1)[:, :Sk][None, None]   # [1, 1, r, Sk]
+            allow = tm if allow is None else allow & tm
+        if allow is not None:
+            s = s.masked_fill(~allow, float("-inf"))
         mx = s.amax(dim=-1, keepdim=True)
         mx = torch.where(torch.isfinite(mx), mx, torch.zeros_like(mx))
         p = torch.exp(s - mx)
@@ -191,7 +204,8 @@ def reference_layer(
     ``bf16_operands`` rounds the normed/rotated K, and the normed/rotated Q times
     ``scale * log2(e)`` (the factor a log2-domain kernel carries in its Q operand), to bf16 first: the
     precision a bf16 matrix unit sees.  Used where logits are so large that this rounding alone
-    exceeds the bf16 tolerance."""
+    exceeds the bf16 tolerance.  Everything runs on the device the inputs live on (the host in the
+    CPU tests; the GPU box's card for the full-size, full-tensor parity tests)."""
     qf, kf = q.to(torch.float64), k.to(torch.float64)
     if q_norm_weight is not None:
         qf = rms_norm(qf, q_norm_weight, norm_eps)

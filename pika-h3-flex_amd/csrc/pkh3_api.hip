@@ -1,6 +1,7 @@
 // C ABI of libpkh3attn.so: argument validation (host only, before any HIP call), workspace
 // planning, and the sequence of launches that makes up one attention call.
 #include "../../include/pkh3_attn.h"
+#include "../../include/pkh3_attn_bench.h"
 
 #include <math.h>
 #include <stdarg.h>
@@ -95,6 +96,7 @@ WsPlan plan(const pkh3_attn_args* a) {
 
 struct Launch {
   WsPlan w;
+  char* ws;  // scratch of this call: the caller's workspace, or the library's static array
   QkPrologueParams kp;
   VPrologueParams vp;
   FwdParams f;
@@ -102,10 +104,11 @@ struct Launch {
   int* idx;
 };
 
-void build(const pkh3_attn_args* a, Launch& L) {
+void build(const pkh3_attn_args* a, void* workspace, Launch& L) {
   const bool fp8 = a->flags & PKH3_FLAG_FP8_QK;
   L.w = plan(a);
-  char* ws = (char*)a->workspace;
+  L.ws = (char*)workspace;
+  char* ws = L.ws;
   L.cnt = a->key_mask ? (int*)(ws + L.w.cnt_off) : nullptr;
   L.idx = a->key_mask ? (int*)(ws + L.w.idx_off) : nullptr;
   const int kBytes = fp8 ? kK8TileBytes : kKTileBytes;
@@ -157,7 +160,7 @@ int run_prologue(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
     if ((e = launch_mask_compact(a->key_mask, a->B, a->Sk, L.idx, L.cnt, st)) != hipSuccess) return hip_fail(e, "mask_compact");
   }
   if (a->blk_row_ptr) {
-    char* ws = (char*)a->workspace;
+    char* ws = L.ws;
     if ((e = launch_sparse_plan(a->blk_row_ptr, a->blk_col_idx, (a->Sq + 63) / 64, L.w.nQ64, L.w.nKt, (int*)(ws + L.w.plan_off),
                                 5 * L.w.nKt, (int*)(ws + L.w.plan_cnt_off), st)) != hipSuccess)
       return hip_fail(e, "sparse plan");
@@ -201,7 +204,7 @@ int pkh3_attn_fwd(const pkh3_attn_args* a, void* stream) {
   int rc = validate(a, true);
   if (rc) return rc;
   Launch L;
-  build(a, L);
+  build(a, a->workspace, L);
   if (a->workspace_bytes < L.w.total)
     return fail(PKH3_EWORKSPACE, "workspace too small: %zu < %zu bytes", a->workspace_bytes, L.w.total);
   hipStream_t st = (hipStream_t)stream;
@@ -218,7 +221,7 @@ int pkh3_attn_time_kernel(const pkh3_attn_args* a, void* stream, int iters, floa
   int rc = validate(a, true);
   if (rc) return rc;
   Launch L;
-  build(a, L);
+  build(a, a->workspace, L);
   if (a->workspace_bytes < L.w.total)
     return fail(PKH3_EWORKSPACE, "workspace too small: %zu < %zu bytes", a->workspace_bytes, L.w.total);
   hipStream_t st = (hipStream_t)stream;

@@ -32,6 +32,8 @@
 // Phase 1 walks the key tiles all four row-blocks keep, exactly like the dense kernel.  Phase 2 walks the
 // remaining tiles per row-block: every iteration gives each wave pair one 32-key half of a tile of its own
 // list in its own LDS area, so all 8 waves stay busy.  The lists are built on the device by a plan kernel.
+#include <atomic>
+
 #include "pkh3_common.h"
 #include "pkh3_internal.h"
 
@@ -49,8 +51,11 @@ constexpr float kStaticMaxLimit = 48.0f;  // rows whose |logit| bound is below t
 // Each tile loop ends on an 8-pass MFMA into the O^T accumulators.  The compiler was seen to place the register
 // copies that merge the two loop variants (v_mov_b64 reading the accumulator's last registers) four scalar
 // instructions after that MFMA, before its result is written back; the block-sparse kernel then returned a stale
-// O^T block.  32 idle issue cycles after every loop let the last MFMA retire whatever follows.
-#define PKH3_MFMA_DRAIN() asm volatile("s_nop 15\n\ts_nop 15" ::: "memory")
+// O^T block.  32 idle issue cycles after every loop let the last MFMA retire whatever follows.  The accumulators
+// are operands of the statement, so every read or copy of them the compiler emits after the loop is ordered
+// after the idle cycles.
+#define PKH3_MFMA_DRAIN(W) \
+  asm volatile("s_nop 15\n\ts_nop 15" : "+v"((W).o[0]), "+v"((W).o[1]), "+v"((W).o[2]), "+v"((W).o[3])::"memory")
 constexpr int kSgMfma = 0x008, kSgDsRead = 0x100;
 
 __device__ __forceinline__ void lds_dma16(const char* g, unsigned lane_off, char* l) {
@@ -64,7 +69,7 @@ __device__ __forceinline__ void lds_dma16(const char* g, unsigned lane_off, char
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
                : "v"(lane_off), "s"(g), "s"(lds_addr)
-               : "memory");
+               : "memory", "m0");
 }
 
 // Wave-uniform reads of tables earlier kernels wrote (tile lists, fp8 scales): through the scalar cache, so
@@ -567,11 +572,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
     if (static_max) {
       PKH3_SHORT_LOOP(true, true, 0, n_lead)
       PKH3_SHORT_LOOP(true, false, n_lead, n_iter)
-      PKH3_MFMA_DRAIN();
+      PKH3_MFMA_DRAIN(w);
     } else {
       PKH3_SHORT_LOOP(false, true, 0, n_lead)
       PKH3_SHORT_LOOP(false, false, n_lead, n_iter)
-      PKH3_MFMA_DRAIN();
+      PKH3_MFMA_DRAIN(w);
     }
     if constexpr (SPLIT) {
       // Add the groups' partial results into group 0, one group at a time through LDS.  On the bounded-logit
@@ -618,11 +623,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
   } else if (static_max) {
     PKH3_TILE_LOOP(true, false, 0, nt - n_masked)
     PKH3_TILE_LOOP(true, true, nt - n_masked, nt)
-    PKH3_MFMA_DRAIN();
+    PKH3_MFMA_DRAIN(w);
   } else {
     PKH3_TILE_LOOP(false, false, 0, nt - n_masked)
     PKH3_TILE_LOOP(false, true, nt - n_masked, nt)
-    PKH3_MFMA_DRAIN();
+    PKH3_MFMA_DRAIN(w);
   }
 #undef PKH3_TILE_LOOP
 #undef PKH3_SHORT_LOOP
@@ -669,10 +674,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
   }
     if (static_max) {
       PKH3_HALF_LOOP(true)
-      PKH3_MFMA_DRAIN();
+      PKH3_MFMA_DRAIN(w);
     } else {
       PKH3_HALF_LOOP(false)
-      PKH3_MFMA_DRAIN();
+      PKH3_MFMA_DRAIN(w);
     }
 #undef PKH3_HALF_LOOP
   }
@@ -738,18 +743,20 @@ static void launch_fp(const FwdParams& p, int cus, hipStream_t st) {
 }
 
 hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
-  // CUs of the current device, asked once per device
-  static int cu_count[64] = {};
+  // CUs of the current device, asked once per device; threads that race here store the same value
+  static std::atomic<int> cu_count[64];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  if (dev >= 0 && dev < 64 && cu_count[dev] == 0) {
-    int n = 0;
-    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return e;
-    cu_count[dev] = n;
+  int cus = 0;
+  if (dev >= 0 && dev < 64) {
+    cus = cu_count[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+      e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      if (e != hipSuccess) return e;
+      cu_count[dev].store(cus, std::memory_order_relaxed);
+    }
   }
-  const int cus = dev >= 0 && dev < 64 ? cu_count[dev] : 0;
   if (p.fp8) launch_fp<true>(p, cus, st);
   else launch_fp<false>(p, cus, st);
   return hipGetLastError();

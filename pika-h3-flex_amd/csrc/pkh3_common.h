@@ -86,7 +86,9 @@ __device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform
 #pragma unroll
     for (int i = 0; i < 64; ++i) ssq += x[i] * x[i];
     ssq += xhalf(ssq);
-    const float rs = rsqrtf(ssq * (1.0f / kD) + t.eps);
+    // an all-zero row with eps == 0 stays all zero instead of 0 * inf
+    const float ms = ssq * (1.0f / kD) + t.eps;
+    const float rs = ms > 0.f ? rsqrtf(ms) : 0.f;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       const f32x4 w0 = *(const f32x4*)(t.norm_w + 16 * ks + 8 * hh);

@@ -21,6 +21,7 @@ class BlockMask:
 
     row_ptr: torch.Tensor  # [ceil(Sq/64)+1]
     col_idx: torch.Tensor  # [nnz]
+    n_cols: Optional[int] = None  # key tiles of the map it was built from (checked against ceil(Sk/64) when known)
 
     @staticmethod
     def from_dense(tile_map: torch.Tensor, device=None) -> "BlockMask":
@@ -33,7 +34,7 @@ class BlockMask:
         if col_idx.numel() == 0:
             col_idx = torch.zeros(1, dtype=torch.int32)
         dev = device if device is not None else tile_map.device
-        return BlockMask(row_ptr.to(dev), col_idx.to(dev))
+        return BlockMask(row_ptr.to(dev), col_idx.to(dev), int(tm.shape[1]))
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -51,11 +52,18 @@ def _check_bshd(name: str, t: torch.Tensor) -> None:
         raise ValueError(f"{name} must live in device memory (got {t.device}); the HIP library is the only compute path")
 
 
-def _f32(name: str, t: Optional[torch.Tensor], shape) -> Optional[torch.Tensor]:
+def _on_device(name: str, t: torch.Tensor, device) -> None:
+    """Every pointer handed to the library is dereferenced by a kernel running on ``device``."""
+    if t.device != device:
+        raise ValueError(f"{name} must live in device memory on {device} (got {t.device})")
+
+
+def _f32(name: str, t: Optional[torch.Tensor], shape, device) -> Optional[torch.Tensor]:
     if t is None:
         return None
     if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != tuple(shape):
         raise ValueError(f"{name} must be contiguous float32 {tuple(shape)}, got {t.dtype} {tuple(t.shape)}")
+    _on_device(name, t, device)
     return t
 
 
@@ -73,6 +81,9 @@ def fill_args(
         raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
     if tuple(out.shape) != (B, Sq, H, D):
         raise ValueError(f"out shape {tuple(out.shape)} != {(B, Sq, H, D)}")
+    dev = q.device
+    for n, t in (("k", k), ("v", v), ("out", out)):
+        _on_device(n, t, dev)
     keep = [q, k, v, out]
     a = _lib.AttnArgs()
     a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
@@ -82,8 +93,8 @@ def fill_args(
     a.o_sb, a.o_ss, a.o_sh = out.stride(0), out.stride(1), out.stride(2)
     a.B, a.H, a.Sq, a.Sk, a.D = B, H, Sq, Sk, D
     a.softmax_scale = float(softmax_scale) if softmax_scale is not None else 0.0
-    qw = _f32("q_norm_weight", q_norm_weight, (D,))
-    kw = _f32("k_norm_weight", k_norm_weight, (D,))
+    qw = _f32("q_norm_weight", q_norm_weight, (D,), dev)
+    kw = _f32("k_norm_weight", k_norm_weight, (D,), dev)
     a.q_norm_w, a.k_norm_w, a.norm_eps = _ptr(qw), _ptr(kw), float(norm_eps)
     a.rope_mode = int(rope_mode)
     if rope_mode != _lib.ROPE_NONE:
@@ -93,13 +104,14 @@ def fill_args(
             if Sq != Sk:
                 raise ValueError("rope_k tables are required when Sq != Sk")
             rope_k = rope_q
-        qc, qs = _f32("rope_q cos", rope_q[0], (Sq, D // 2)), _f32("rope_q sin", rope_q[1], (Sq, D // 2))
-        kc, ks = _f32("rope_k cos", rope_k[0], (Sk, D // 2)), _f32("rope_k sin", rope_k[1], (Sk, D // 2))
+        qc, qs = _f32("rope_q cos", rope_q[0], (Sq, D // 2), dev), _f32("rope_q sin", rope_q[1], (Sq, D // 2), dev)
+        kc, ks = _f32("rope_k cos", rope_k[0], (Sk, D // 2), dev), _f32("rope_k sin", rope_k[1], (Sk, D // 2), dev)
         a.q_rope_cos, a.q_rope_sin, a.k_rope_cos, a.k_rope_sin = qc.data_ptr(), qs.data_ptr(), kc.data_ptr(), ks.data_ptr()
         keep += [qc, qs, kc, ks]
     if key_mask is not None:
         if tuple(key_mask.shape) != (B, Sk):
             raise ValueError(f"key_mask must be [B, Sk] = {(B, Sk)}, got {tuple(key_mask.shape)}")
+        _on_device("key_mask", key_mask, dev)
         km = key_mask.to(torch.uint8).contiguous() if key_mask.dtype != torch.uint8 else key_mask.contiguous()
         a.key_mask = km.data_ptr()
         keep.append(km)
@@ -109,6 +121,12 @@ def fill_args(
             raise TypeError("block mask CSR arrays must be int32")
         if block_mask.row_ptr.numel() != nrow + 1:
             raise ValueError(f"block mask has {block_mask.row_ptr.numel() - 1} tile rows, need {nrow}")
+        if block_mask.n_cols is not None and block_mask.n_cols != (Sk + 63) // 64:
+            raise ValueError(f"block mask has {block_mask.n_cols} tile columns, need {(Sk + 63) // 64}")
+        _on_device("block mask row_ptr", block_mask.row_ptr, dev)
+        _on_device("block mask col_idx", block_mask.col_idx, dev)
+        if not (block_mask.row_ptr.is_contiguous() and block_mask.col_idx.is_contiguous()):
+            raise ValueError("block mask CSR arrays must be contiguous")
         a.blk_row_ptr, a.blk_col_idx = block_mask.row_ptr.data_ptr(), block_mask.col_idx.data_ptr()
         keep += [block_mask.row_ptr, block_mask.col_idx]
     a.flags = (_lib.FLAG_FP8_QK if fp8_qk else 0) | (_lib.FLAG_LONG_KEY_KERNEL if long_key_kernel else 0)
@@ -125,25 +143,30 @@ def workspace_bytes(args: _lib.AttnArgs) -> int:
 
 def attention(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, out: Optional[torch.Tensor] = None,
-    workspace: Optional[torch.Tensor] = None, **opts,
+    workspace=None, **opts,
 ) -> torch.Tensor:
     """softmax(norm_rope(q) norm_rope(k)^T * scale) v over ``[B, S, H, D]`` bf16 views (any strides
-    with a unit head-dim stride).  Keyword options are those of :func:`fill_args`.  Runs
-    asynchronously on the current stream and returns ``out`` ([B, Sq, H, D], bf16)."""
+    with a unit head-dim stride).  Keyword options are those of :func:`fill_args`.  ``workspace`` is a
+    uint8 device tensor to use as scratch when large enough, or a callable ``(device, nbytes) -> tensor``
+    that provides one; without it a fresh buffer is allocated.  Runs asynchronously on the current stream and returns ``out`` ([B, Sq, H, D], bf16)."""
     lib = _lib.load()
     if out is None:
         out = torch.empty((q.shape[0], q.shape[1], q.shape[2], q.shape[3]), dtype=torch.bfloat16, device=q.device)
     args, keep = fill_args(q, k, v, out, **opts)
     need = workspace_bytes(args)
+    if callable(workspace):
+        workspace = workspace(q.device, need)
     if workspace is None or workspace.numel() * workspace.element_size() < need:
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
     args.workspace = workspace.data_ptr()
     args.workspace_bytes = workspace.numel() * workspace.element_size()
+    if workspace.device != q.device:
+        raise ValueError(f"workspace must live on {q.device} (got {workspace.device})")
     with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream().cuda_stream
-        _lib.check(lib.pkh3_attn_fwd(C.byref(args), C.c_void_p(stream)))
-    # the workspace must outlive the kernels: tie it to the stream, not to this Python frame
-    workspace.record_stream(torch.cuda.current_stream())
+        stream = torch.cuda.current_stream()
+        _lib.check(lib.pkh3_attn_fwd(C.byref(args), C.c_void_p(stream.cuda_stream)))
+        # the workspace must outlive the kernels: tie it to the stream, not to this Python frame
+        workspace.record_stream(stream)
     return out
 
 

@@ -14,7 +14,7 @@ RoPE pairing (``rope_mode``), axis split and theta, and where the norm weights a
 """
 from __future__ import annotations
 
-from typing import Dict, Optional, Tuple
+from typing import Dict, Hashable, Optional, Tuple
 
 import torch
 
@@ -56,18 +56,37 @@ class PikaH3AttnProcessor:
         self.norm_eps = float(norm_eps)
         self.fp8_qk = bool(fp8_qk)
         # position grids are constant across layers and denoising steps: one table per grid
-        self._rope_cache: Dict[Tuple[int, int, str], Tuple[torch.Tensor, torch.Tensor]] = {}
-        self._workspace: Optional[torch.Tensor] = None
+        self._rope_cache: Dict[Hashable, Tuple[Optional[torch.Tensor], Tuple[torch.Tensor, torch.Tensor]]] = {}
+        # one scratch buffer per (device, stream), grown on demand and reused by every layer call on that stream
+        self._workspaces: Dict[Tuple[str, int], torch.Tensor] = {}
 
-    def _tables(self, position_ids: torch.Tensor):
-        key = (position_ids.data_ptr(), position_ids.shape[0], str(position_ids.device))
+    def _tables(self, position_ids: torch.Tensor, rope_key: Optional[Hashable] = None):
+        """cos/sin tables of a position grid, cached.  With ``rope_key`` (e.g. the caller's geometry key) the cache
+        is keyed by it and the grid's identity does not matter.  Without, the key is the grid tensor itself --
+        address, length, device and in-place version counter -- and the entry keeps the tensor alive, so its
+        address cannot be handed to another grid while the entry exists."""
+        if rope_key is not None:
+            key = ("key", rope_key, position_ids.shape[0], str(position_ids.device))
+        else:
+            key = ("tensor", position_ids.data_ptr(), position_ids.shape[0], str(position_ids.device),
+                   position_ids._version)
         hit = self._rope_cache.get(key)
         if hit is None:
             if len(self._rope_cache) >= 8:
                 self._rope_cache.pop(next(iter(self._rope_cache)))
-            hit = rope_tables(position_ids, self.rope_axes_dims, self.rope_theta)
+            tabs = rope_tables(position_ids, self.rope_axes_dims, self.rope_theta)
+            hit = (position_ids if rope_key is None else None, tabs)
             self._rope_cache[key] = hit
-        return hit
+        return hit[1]
+
+    def _workspace(self, device, nbytes: int) -> torch.Tensor:
+        with torch.cuda.device(device):
+            key = (str(device), int(torch.cuda.current_stream().cuda_stream))
+        ws = self._workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self._workspaces[key] = ws
+        return ws
 
     def __call__(
         self,
@@ -80,13 +99,16 @@ class PikaH3AttnProcessor:
         rope_cos_sin: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
         block_mask: Optional[BlockMask] = None,
         fp8_qk: Optional[bool] = None,
+        rope_key: Optional[Hashable] = None,
     ) -> torch.Tensor:
         """``hidden_states [B, S, H*D]`` -> ``[B, S, H*D]``.
 
         Self-attention when ``encoder_hidden_states`` is None, else cross-attention with K/V from
         ``encoder_hidden_states [B, Sk, C]`` and ``attention_mask`` a bool key-padding mask
         ``[B, Sk]`` (True = attend).  RoPE applies to self-attention only, from ``position_ids
-        [S, 3]`` (or precomputed ``rope_cos_sin`` fp32 ``[S, D/2]`` tables).
+        [S, 3]`` (or precomputed ``rope_cos_sin`` fp32 ``[S, D/2]`` tables); ``rope_key`` names the grid for the
+        table cache (see :meth:`_tables`).  The softmax scale is ``attn.scale`` when the module has one, else
+        ``1/sqrt(D)``.  fp8 QK^T is not defined together with a key mask: such a call runs in bf16.
         """
         if hidden_states.dim() != 3:
             raise ValueError(f"hidden_states must be [B, S, C], got {tuple(hidden_states.shape)}")
@@ -105,17 +127,21 @@ class PikaH3AttnProcessor:
             q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
 
         qn, kn = getattr(attn, "norm_q", None), getattr(attn, "norm_k", None)
-        eps = float(getattr(qn, "eps", None) or self.norm_eps)
+        eps = getattr(qn, "eps", None)
+        eps = self.norm_eps if eps is None else float(eps)
+        scale = getattr(attn, "scale", None)
+        use_fp8 = (self.fp8_qk if fp8_qk is None else bool(fp8_qk)) and attention_mask is None
         opts = dict(
             q_norm_weight=_norm_weight(qn, D, q.device),
             k_norm_weight=_norm_weight(kn, D, q.device),
             norm_eps=eps,
-            fp8_qk=self.fp8_qk if fp8_qk is None else bool(fp8_qk),
+            fp8_qk=use_fp8,
             block_mask=block_mask,
+            softmax_scale=None if scale is None else float(scale),
         )
         if encoder_hidden_states is None:
             if rope_cos_sin is None and position_ids is not None:
-                rope_cos_sin = self._tables(position_ids)
+                rope_cos_sin = self._tables(position_ids, rope_key)
             if rope_cos_sin is not None:
                 opts.update(rope_mode=self.rope_mode, rope_q=rope_cos_sin, rope_k=rope_cos_sin)
             if attention_mask is not None:
@@ -124,8 +150,7 @@ class PikaH3AttnProcessor:
             if attention_mask is not None:
                 opts.update(key_mask=attention_mask)
 
-        need_ws = self._workspace
-        out = attention(q, k, v, workspace=need_ws, **opts)
+        out = attention(q, k, v, workspace=self._workspace, **opts)
         out = out.view(B, S, H * D).to(hidden_states.dtype)
         out = attn.to_out[0](out)
         if len(attn.to_out) > 1:

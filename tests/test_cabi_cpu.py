@@ -13,7 +13,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def test_header_symbols_are_exported(lib):
-    header = open(os.path.join(ROOT, "include", "pkh3_attn.h")).read()
+    inc = os.path.join(ROOT, "include")
+    header = "".join(open(os.path.join(inc, f)).read() for f in sorted(os.listdir(inc)) if f.endswith(".h"))
     declared = set(re.findall(r"\b(pkh3_[a-z0-9_]+)\s*\(", header))
     assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
     for name in declared:
@@ -119,6 +120,24 @@ def test_time_kernel_argument_errors(lib):
     assert lib.pkh3_attn_time_kernel(C.byref(a), None, 1, None) == _lib.PKH3_ENULL
     ms = C.c_float()
     assert lib.pkh3_attn_time_kernel(C.byref(a), None, 0, C.byref(ms)) == _lib.PKH3_EARG
+
+
+def test_front_end_checks_every_pointer_for_its_device():
+    """Tensors handed over by address (norm weights, rope tables, masks) must live where the kernels run."""
+    import torch
+
+    from pika_h3_flex_amd import ops
+
+    host = torch.ones(128)
+    with pytest.raises(ValueError, match="device memory"):
+        ops._f32("q_norm_weight", host, (128,), torch.device("meta"))
+    assert ops._f32("w", host, (128,), torch.device("cpu")) is host
+    with pytest.raises(ValueError, match="contiguous float32"):
+        ops._f32("w", host.double(), (128,), torch.device("cpu"))
+    with pytest.raises(ValueError, match="device memory"):
+        ops._on_device("key_mask", torch.zeros(4, dtype=torch.bool), torch.device("meta"))
+    bm = ops.BlockMask.from_dense(torch.ones((2, 3), dtype=torch.bool), device="cpu")
+    assert bm.n_cols == 3
 
 
 def test_ops_refuse_host_tensors():

@@ -221,6 +221,13 @@ def test_fp8_round_agrees_with_torch_cast():
     x = np.concatenate([rng.uniform(-448, 448, 5000), rng.normal(0, 2, 5000)]).astype(np.float32)
     ref = torch.from_numpy(x).to(torch.float8_e4m3fn).to(torch.float64).numpy()
     assert np.array_equal(O.fp8_e4m3_round(x.astype(np.float64)), ref)
+    # the device-side variant of the rounding (used when the oracle runs on the GPU box's card) is that cast
+    assert np.array_equal(O.fp8_e4m3_round_torch(torch.from_numpy(x)).numpy(), ref)
+    # ... including every representable value, the extremes and values just below/above the midpoints
+    grid = np.array(sorted({_decode_e4m3fn(c) for c in range(256) if not math.isnan(_decode_e4m3fn(c))}), dtype=np.float32)
+    mids = ((grid[1:] + grid[:-1]) / 2).astype(np.float32)
+    probe = np.concatenate([grid, mids, np.nextafter(mids, np.float32(1e9)), np.nextafter(mids, np.float32(-1e9))])
+    assert np.array_equal(O.fp8_e4m3_round_torch(torch.from_numpy(probe)).numpy(), O.fp8_e4m3_round(probe.astype(np.float64)))
 
 
 def test_fake_quant_blocks_scales_and_error_bound():
