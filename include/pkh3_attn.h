@@ -115,6 +115,18 @@ size_t pkh3_workspace_bytes(const pkh3_attn_args* a);
    the output projection (module at src/pika_h3/core/loader.py:9; call site src/pika_h3/core/wrapper.py:248). */
 int pkh3_attn_fwd(const pkh3_attn_args* a, void* stream);
 
+/* The same call for callers that cannot allocate device memory or pass a workspace (code under HIP graph
+   capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+   `workspace` / `workspace_bytes` of `a` are ignored: the scratch is an array built into the library, one
+   copy per GPU, PKH3_NOALLOC_SCRATCH_BYTES long, held until the process ends.  The call allocates and frees
+   nothing.  Calls whose pkh3_workspace_bytes() exceeds that size are rejected with PKH3_EWORKSPACE.  Every
+   call on one GPU shares that GPU's array (each call rewrites all of it that it reads, so nothing needs
+   clearing between calls), hence two such calls that may overlap on one GPU -- different streams, or one
+   graph launched twice at once -- race; calls on one stream are ordered and safe.  Same kernels, same
+   results as pkh3_attn_fwd. */
+#define PKH3_NOALLOC_SCRATCH_BYTES (64u << 20)
+int pkh3_attn_fwd_noalloc(const pkh3_attn_args* a, void* stream);
+
 /* Rotary tables from the packed layout's position grid (src/pika_h3/core/packing.py:128 position_ids
    [S,3] float64, device memory).  axis_dims[3] are the head-dim slices per (t,h,w) axis (sum = D,
    each even); pair p of axis a rotates by pos[a] * theta^(-2*i/axis_dims[a]) with i the pair's index

@@ -25,10 +25,12 @@ PKH3_EARG = -9
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_HALF = 0, 1, 2
 FLAG_FP8_QK = 1
 FLAG_LONG_KEY_KERNEL = 2
+NOALLOC_SCRATCH_BYTES = 64 << 20  # PKH3_NOALLOC_SCRATCH_BYTES
 
 EXPORTS = (
     "pkh3_workspace_bytes",
     "pkh3_attn_fwd",
+    "pkh3_attn_fwd_noalloc",
     "pkh3_rope_tables",
     "pkh3_version",
     "pkh3_strerror",
@@ -85,6 +87,8 @@ def load() -> C.CDLL:
     lib.pkh3_workspace_bytes.restype = C.c_size_t
     lib.pkh3_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
     lib.pkh3_attn_fwd.restype = C.c_int
+    lib.pkh3_attn_fwd_noalloc.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
+    lib.pkh3_attn_fwd_noalloc.restype = C.c_int
     lib.pkh3_attn_time_kernel.argtypes = [C.POINTER(AttnArgs), C.c_void_p, C.c_int, C.POINTER(C.c_float)]
     lib.pkh3_attn_time_kernel.restype = C.c_int
     lib.pkh3_rope_tables.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_int32), C.c_double, C.c_void_p, C.c_void_p, C.c_void_p]

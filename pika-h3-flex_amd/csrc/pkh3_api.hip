@@ -4,6 +4,8 @@
 #include "../../include/pkh3_attn_bench.h"
 
 #include <math.h>
+
+#include <mutex>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -40,8 +42,9 @@ int check_tensor(const char* name, const void* ptr, int64_t sb, int64_t ss, int6
   return PKH3_OK;
 }
 
-// Validation shared by pkh3_workspace_bytes (shapes/options only) and pkh3_attn_fwd (everything).
-int validate(const pkh3_attn_args* a, bool pointers) {
+// Validation shared by pkh3_workspace_bytes (shapes/options only), pkh3_attn_fwd (everything) and
+// pkh3_attn_fwd_noalloc (everything but the caller's workspace, which it does not use).
+int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = true) {
   if (!a) return fail(PKH3_ENULL, "args is NULL");
   if (a->D != kD) return fail(PKH3_EHEADDIM, "head dim must be 128, got %d", a->D);
   if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Sk < 1) return fail(PKH3_ESHAPE, "B, H, Sq, Sk must be >= 1");
@@ -70,6 +73,7 @@ int validate(const pkh3_attn_args* a, bool pointers) {
   }
   if ((a->q_norm_w && misaligned16(a->q_norm_w)) || (a->k_norm_w && misaligned16(a->k_norm_w)))
     return fail(PKH3_EALIGN, "norm weights must be 16-byte aligned");
+  if (!caller_workspace) return PKH3_OK;
   if (!a->workspace) return fail(PKH3_EWORKSPACE, "workspace is NULL");
   if ((uintptr_t)a->workspace & 255u) return fail(PKH3_EWORKSPACE, "workspace is not 256-byte aligned");
   return PKH3_OK;
@@ -171,6 +175,32 @@ int run_prologue(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
   return PKH3_OK;
 }
 
+// Scratch of pkh3_attn_fwd_noalloc: one array per GPU the library is loaded on, held until the process ends.
+// In host code the array's name is only a handle; each device's copy has its own address, looked up once per
+// device (with that device current) and used from then on wherever the memory itself is meant.
+static __device__ __align__(256) unsigned char scratch[PKH3_NOALLOC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(PKH3_EARG, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    if (!ptr || ((uintptr_t)ptr & 255u)) return fail(PKH3_EHIP, "built-in scratch buffer has an unusable address");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return PKH3_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -207,6 +237,27 @@ int pkh3_attn_fwd(const pkh3_attn_args* a, void* stream) {
   build(a, a->workspace, L);
   if (a->workspace_bytes < L.w.total)
     return fail(PKH3_EWORKSPACE, "workspace too small: %zu < %zu bytes", a->workspace_bytes, L.w.total);
+  hipStream_t st = (hipStream_t)stream;
+  if ((rc = run_prologue(a, L, st))) return rc;
+  hipError_t e = launch_attn_fwd(L.f, st);
+  if (e != hipSuccess) return hip_fail(e, "attn_fwd");
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
+int pkh3_attn_fwd_noalloc(const pkh3_attn_args* a, void* stream) {
+  int rc = validate(a, true, /*caller_workspace=*/false);
+  if (rc) return rc;
+  const size_t need = plan(a).total;
+  if (need > (size_t)PKH3_NOALLOC_SCRATCH_BYTES)
+    return fail(PKH3_EWORKSPACE,
+                "pkh3_attn_fwd_noalloc: this call needs %zu bytes of scratch, the built-in buffer holds %zu; use "
+                "pkh3_attn_fwd with a caller-owned workspace",
+                need, (size_t)PKH3_NOALLOC_SCRATCH_BYTES);
+  void* ptr = nullptr;  // this device's copy of the built-in scratch array
+  if ((rc = static_scratch(&ptr))) return rc;
+  Launch L;
+  build(a, ptr, L);
   hipStream_t st = (hipStream_t)stream;
   if ((rc = run_prologue(a, L, st))) return rc;
   hipError_t e = launch_attn_fwd(L.f, st);

@@ -143,16 +143,23 @@ def workspace_bytes(args: _lib.AttnArgs) -> int:
 
 def attention(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, out: Optional[torch.Tensor] = None,
-    workspace=None, **opts,
+    workspace=None, static_scratch: bool = False, **opts,
 ) -> torch.Tensor:
     """softmax(norm_rope(q) norm_rope(k)^T * scale) v over ``[B, S, H, D]`` bf16 views (any strides
     with a unit head-dim stride).  Keyword options are those of :func:`fill_args`.  ``workspace`` is a
     uint8 device tensor to use as scratch when large enough, or a callable ``(device, nbytes) -> tensor``
-    that provides one; without it a fresh buffer is allocated.  Runs asynchronously on the current stream and returns ``out`` ([B, Sq, H, D], bf16)."""
+    that provides one; without it a fresh buffer is allocated.  ``static_scratch=True`` calls the
+    entry point that allocates nothing instead (``pkh3_attn_fwd_noalloc``: scratch built into the library,
+    at most ``_lib.NOALLOC_SCRATCH_BYTES``; pass ``out`` as well and the call touches no allocator at all).
+    Runs asynchronously on the current stream and returns ``out`` ([B, Sq, H, D], bf16)."""
     lib = _lib.load()
     if out is None:
         out = torch.empty((q.shape[0], q.shape[1], q.shape[2], q.shape[3]), dtype=torch.bfloat16, device=q.device)
     args, keep = fill_args(q, k, v, out, **opts)
+    if static_scratch:
+        with torch.cuda.device(q.device):
+            _lib.check(lib.pkh3_attn_fwd_noalloc(C.byref(args), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        return out
     need = workspace_bytes(args)
     if callable(workspace):
         workspace = workspace(q.device, need)

@@ -122,6 +122,27 @@ def test_time_kernel_argument_errors(lib):
     assert lib.pkh3_attn_time_kernel(C.byref(a), None, 0, C.byref(ms)) == _lib.PKH3_EARG
 
 
+def test_noalloc_entry_point_validates_on_the_host(lib):
+    """pkh3_attn_fwd_noalloc ignores the caller's workspace fields, checks everything else like pkh3_attn_fwd,
+    and rejects a call whose scratch would not fit its built-in buffer -- all before any HIP call."""
+    a = _valid_args()
+    a.q = 0
+    assert lib.pkh3_attn_fwd_noalloc(C.byref(a), None) == _lib.PKH3_ENULL
+    a = _valid_args()
+    a.D = 64
+    assert lib.pkh3_attn_fwd_noalloc(C.byref(a), None) == _lib.PKH3_EHEADDIM
+    a = _valid_args()
+    a.workspace, a.workspace_bytes = 0, 0       # not an error here
+    a.H, a.Sk = 24, 8192                        # 24 x 128 tiles x 32 KiB = 96 MiB of K/V images
+    for n in ("q", "k", "v", "o"):
+        setattr(a, n + "_ss", 24 * 128)
+    assert lib.pkh3_workspace_bytes(C.byref(a)) > _lib.NOALLOC_SCRATCH_BYTES
+    assert lib.pkh3_attn_fwd_noalloc(C.byref(a), None) == _lib.PKH3_EWORKSPACE
+    assert b"built-in" in lib.pkh3_last_error()
+    header = open(os.path.join(ROOT, "include", "pkh3_attn.h")).read()
+    assert re.search(r"#define\s+PKH3_NOALLOC_SCRATCH_BYTES\s+\(64u\s*<<\s*20\)", header)
+
+
 def test_front_end_checks_every_pointer_for_its_device():
     """Tensors handed over by address (norm weights, rope tables, masks) must live where the kernels run."""
     import torch
