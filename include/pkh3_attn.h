@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define PKH3_VERSION 101
+#define PKH3_VERSION 102
 
 enum {
   PKH3_OK = 0,
@@ -65,6 +65,9 @@ enum {
 enum {
   PKH3_FLAG_FP8_QK = 1u << 0, /* quantise normed+roped Q and K to fp8 e4m3 (OCP) with one absmax scale
                                  per (batch, head, 64-row block); P.V stays bf16 with fp32 accumulation */
+  PKH3_FLAG_KV_PREPARED = 1u << 2, /* K and V already lie in `workspace` as the attention kernel reads them, written
+                                 there by pkh3_qkv_proj on the same stream with the same shapes and options: the
+                                 call skips its own K/V pass; `k` and `v` are not read and may be NULL */
   PKH3_FLAG_LONG_KEY_KERNEL = 1u << 1 /* dense calls with at most 16 key tiles (Sk <= 1024) normally run a
                                  short-key form of the kernel (small workgroups, three per CU); this flag
                                  selects the long-key form for them too.  Same results to the tolerance of the
@@ -133,6 +136,88 @@ int pkh3_attn_fwd_noalloc(const pkh3_attn_args* a, void* stream);
    inside its axis slice.  Writes cos/sin fp32 [S, D/2]. */
 int pkh3_rope_tables(const double* position_ids, int32_t S, const int32_t axis_dims[3], double theta,
                      float* cos_out, float* sin_out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------
+ * Projections around the attention call: the `to_q / to_k / to_v / to_out.0` linear layers of the
+ * attention module with their LoRA adapters (target list src/pika_h3/core/loader.py:9, rank/alpha
+ * injection src/pika_h3/core/loader.py:20-49, applied at src/pika_h3/pipeline.py:105-107) and the AdaLN
+ * modulation that feeds them (patches/0001-h3-adaln-fp32.patch:34-40: norm(x) * (1 + scale[idx]) +
+ * shift[idx], rows gathered by `timestep_indices`, src/pika_h3/core/wrapper.py:182-190,196-197).
+ *
+ * Matrix operands are kept as "operand images": 1 KiB blocks of 32 rows x 16 contraction elements in
+ * the register order of the gfx950 32x32x16 MFMA.  Weights are packed once (pkh3_pack_weight) when
+ * they are loaded; activations are packed by the kernel that produces them (pkh3_adaln_modulate) or
+ * by pkh3_pack_rows.  A packed buffer for [rows, K] takes pkh3_packed_bytes(rows, K) bytes, 256-byte
+ * aligned; rows are padded to a multiple of 256 with zeros.  K must be a multiple of 32 and <= 4096.
+ */
+enum { PKH3_NORM_NONE = 0, PKH3_NORM_LAYER = 1 /* (x - mean) * rsqrt(var + eps), no affine */,
+       PKH3_NORM_RMS = 2 /* x * rsqrt(mean(x^2) + eps), no weight */ };
+
+#define PKH3_LORA_RANK 128 /* the adapters' rank (src/pika_h3/pipeline.py:34 via the manifest); other ranks: PKH3_EUNSUPPORTED */
+
+size_t pkh3_packed_bytes(int32_t rows, int32_t K);
+
+/* W bf16 [N, K] (row = output feature, `row_stride` elements between rows; torch Linear.weight) -> images.
+   N must be a multiple of 128.  head_perm = 1 stores the rows of every 128-feature head in the order the
+   row-per-lane epilogues need (Q, K, to_out.0, LoRA A and the B matrices that go with them); head_perm = 0
+   for a V projection and its LoRA B, whose epilogue holds one feature per lane. */
+int pkh3_pack_weight(const void* w, int64_t row_stride, int32_t N, int32_t K, int32_t head_perm, void* out,
+                     void* stream);
+
+/* x bf16 [S, K] row-major (`row_stride` elements between rows) -> images of the activations. */
+int pkh3_pack_rows(const void* x, int64_t row_stride, int32_t S, int32_t K, void* out, void* stream);
+
+/* AdaLN modulation fused with the packing: out = images of norm(x) * (1 + scale[row_index[s]]) +
+   shift[row_index[s]], statistics and arithmetic in fp32, one rounding to bf16.  shift / scale: bf16
+   [table rows, table_stride] (either may be NULL: no such term); row_index int32 [S] or NULL (table row
+   0 for every token).  Replaces the modulation of patches/0001-h3-adaln-fp32.patch:34-40. */
+int pkh3_adaln_modulate(const void* x, int64_t row_stride, int32_t S, int32_t K, int32_t norm_kind, float eps,
+                        const void* shift, const void* scale, int64_t table_stride, const int32_t* row_index,
+                        void* out, void* stream);
+
+/* One linear layer with its adapter: y = x W^T + bias + lora_scale * (x A^T) B^T. */
+typedef struct pkh3_linear {
+  const void* w_img;       /* pkh3_pack_weight(W [N, K]) */
+  const float* bias;       /* fp32 [N] or NULL */
+  const void* lora_a_img;  /* pkh3_pack_weight(A [PKH3_LORA_RANK, K], head_perm = 1) or NULL: no adapter */
+  const void* lora_b_img;  /* pkh3_pack_weight(B [N, PKH3_LORA_RANK], head_perm as for w_img) */
+  float lora_scale;        /* lora_alpha / rank */
+} pkh3_linear;
+
+typedef struct pkh3_qkv_args {
+  const void* x_img;       /* activations [S, K] as images */
+  int32_t S, K;            /* tokens, hidden size */
+  pkh3_linear q, k, v;     /* N = H * 128 each; q and k packed with head_perm = 1, v with head_perm = 0 */
+  void* lora_workspace;    /* scratch for the down-projected rows: pkh3_packed_bytes(S, 3 * PKH3_LORA_RANK); may be
+                              NULL when no projection has an adapter */
+  size_t lora_workspace_bytes;
+} pkh3_qkv_args;
+
+/* to_q / to_k / to_v of one self-attention call in one launch (plus one for the adapters' down-projection).
+   `attn` describes the attention call that follows (B = 1, Sq = Sk = S, no key mask): Q is written as bf16 to
+   attn->q with attn's strides; K goes through QK-RMSNorm (attn->k_norm_w, norm_eps), rotation (attn->rope_mode,
+   k_rope_cos / k_rope_sin) and, with PKH3_FLAG_FP8_QK, quantisation, and K and V are written into attn->workspace
+   in the layout the attention kernel reads.  Then call pkh3_attn_fwd(attn) with PKH3_FLAG_KV_PREPARED added.
+   attn->k, attn->v and attn->o are not touched by this call. */
+int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* attn, void* stream);
+
+typedef struct pkh3_out_args {
+  const void* o_img;       /* attention output [S, K] as images (pkh3_pack_rows of O viewed as [S, H*128]) */
+  int32_t S, K, N;
+  pkh3_linear proj;        /* packed with head_perm = 1 */
+  const void* gate;        /* bf16 [table rows, gate_stride] or NULL; row_index int32 [S] or NULL (row 0) */
+  int64_t gate_stride;
+  const int32_t* row_index;
+  const void* residual;    /* bf16 [S, residual_stride] or NULL */
+  int64_t residual_stride;
+  void* y;                 /* bf16 [S, y_stride]: residual + gate[row_index] * (o W^T + bias + adapter) */
+  int64_t y_stride;
+  void* lora_workspace;    /* pkh3_packed_bytes(S, PKH3_LORA_RANK) when proj has an adapter */
+  size_t lora_workspace_bytes;
+} pkh3_out_args;
+
+/* to_out.0 with its adapter and the gated residual update of the block around it. */
+int pkh3_out_proj(const pkh3_out_args* p, void* stream);
 
 int pkh3_version(void);
 const char* pkh3_strerror(int code);

@@ -25,6 +25,9 @@ PKH3_EARG = -9
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_HALF = 0, 1, 2
 FLAG_FP8_QK = 1
 FLAG_LONG_KEY_KERNEL = 2
+FLAG_KV_PREPARED = 4
+NORM_NONE, NORM_LAYER, NORM_RMS = 0, 1, 2
+LORA_RANK = 128  # PKH3_LORA_RANK
 NOALLOC_SCRATCH_BYTES = 64 << 20  # PKH3_NOALLOC_SCRATCH_BYTES
 
 EXPORTS = (
@@ -36,6 +39,12 @@ EXPORTS = (
     "pkh3_strerror",
     "pkh3_last_error",
     "pkh3_attn_time_kernel",
+    "pkh3_packed_bytes",
+    "pkh3_pack_weight",
+    "pkh3_pack_rows",
+    "pkh3_adaln_modulate",
+    "pkh3_qkv_proj",
+    "pkh3_out_proj",
 )
 
 
@@ -59,6 +68,39 @@ class AttnArgs(C.Structure):
         ("blk_row_ptr", C.c_void_p), ("blk_col_idx", C.c_void_p),
         ("flags", C.c_uint32),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+    ]
+
+
+class Linear(C.Structure):
+    """Mirror of ``struct pkh3_linear``."""
+
+    _fields_ = [
+        ("w_img", C.c_void_p), ("bias", C.c_void_p),
+        ("lora_a_img", C.c_void_p), ("lora_b_img", C.c_void_p),
+        ("lora_scale", C.c_float),
+    ]
+
+
+class QkvArgs(C.Structure):
+    """Mirror of ``struct pkh3_qkv_args``."""
+
+    _fields_ = [
+        ("x_img", C.c_void_p), ("S", C.c_int32), ("K", C.c_int32),
+        ("q", Linear), ("k", Linear), ("v", Linear),
+        ("lora_workspace", C.c_void_p), ("lora_workspace_bytes", C.c_size_t),
+    ]
+
+
+class OutArgs(C.Structure):
+    """Mirror of ``struct pkh3_out_args``."""
+
+    _fields_ = [
+        ("o_img", C.c_void_p), ("S", C.c_int32), ("K", C.c_int32), ("N", C.c_int32),
+        ("proj", Linear),
+        ("gate", C.c_void_p), ("gate_stride", C.c_int64), ("row_index", C.c_void_p),
+        ("residual", C.c_void_p), ("residual_stride", C.c_int64),
+        ("y", C.c_void_p), ("y_stride", C.c_int64),
+        ("lora_workspace", C.c_void_p), ("lora_workspace_bytes", C.c_size_t),
     ]
 
 
@@ -93,6 +135,19 @@ def load() -> C.CDLL:
     lib.pkh3_attn_time_kernel.restype = C.c_int
     lib.pkh3_rope_tables.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_int32), C.c_double, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.pkh3_rope_tables.restype = C.c_int
+    lib.pkh3_packed_bytes.argtypes = [C.c_int32, C.c_int32]
+    lib.pkh3_packed_bytes.restype = C.c_size_t
+    lib.pkh3_pack_weight.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.pkh3_pack_weight.restype = C.c_int
+    lib.pkh3_pack_rows.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.pkh3_pack_rows.restype = C.c_int
+    lib.pkh3_adaln_modulate.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_void_p,
+                                        C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.pkh3_adaln_modulate.restype = C.c_int
+    lib.pkh3_qkv_proj.argtypes = [C.POINTER(QkvArgs), C.POINTER(AttnArgs), C.c_void_p]
+    lib.pkh3_qkv_proj.restype = C.c_int
+    lib.pkh3_out_proj.argtypes = [C.POINTER(OutArgs), C.c_void_p]
+    lib.pkh3_out_proj.restype = C.c_int
     lib.pkh3_version.argtypes = []
     lib.pkh3_version.restype = C.c_int
     lib.pkh3_strerror.argtypes = [C.c_int]

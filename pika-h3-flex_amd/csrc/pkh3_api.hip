@@ -44,13 +44,16 @@ int check_tensor(const char* name, const void* ptr, int64_t sb, int64_t ss, int6
 
 // Validation shared by pkh3_workspace_bytes (shapes/options only), pkh3_attn_fwd (everything) and
 // pkh3_attn_fwd_noalloc (everything but the caller's workspace, which it does not use).
-int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = true) {
+int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = true, bool need_kv = true) {
   if (!a) return fail(PKH3_ENULL, "args is NULL");
   if (a->D != kD) return fail(PKH3_EHEADDIM, "head dim must be 128, got %d", a->D);
   if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Sk < 1) return fail(PKH3_ESHAPE, "B, H, Sq, Sk must be >= 1");
   if (a->B > 65535 || a->H > 65535) return fail(PKH3_ESHAPE, "B and H must be <= 65535");
   if (a->Sq > (1 << 24) || a->Sk > (1 << 24)) return fail(PKH3_ESHAPE, "Sq and Sk must be <= 2^24");
-  if (a->flags & ~(uint32_t)(PKH3_FLAG_FP8_QK | PKH3_FLAG_LONG_KEY_KERNEL)) return fail(PKH3_EARG, "unknown flag bits 0x%x", a->flags);
+  if (a->flags & ~(uint32_t)(PKH3_FLAG_FP8_QK | PKH3_FLAG_LONG_KEY_KERNEL | PKH3_FLAG_KV_PREPARED))
+    return fail(PKH3_EARG, "unknown flag bits 0x%x", a->flags);
+  if ((a->flags & PKH3_FLAG_KV_PREPARED) && (a->key_mask || a->B != 1 || a->Sq != a->Sk))
+    return fail(PKH3_EUNSUPPORTED, "prepared K/V (pkh3_qkv_proj) means one self-attention document: B = 1, Sq = Sk, no key mask");
   if (a->rope_mode < PKH3_ROPE_NONE || a->rope_mode > PKH3_ROPE_HALF) return fail(PKH3_EARG, "bad rope_mode %d", a->rope_mode);
   if (!(a->softmax_scale == a->softmax_scale) || isinf(a->softmax_scale)) return fail(PKH3_EARG, "softmax_scale is not finite");
   if ((a->q_norm_w || a->k_norm_w) && !(a->norm_eps >= 0.f)) return fail(PKH3_EARG, "norm_eps must be >= 0");
@@ -62,8 +65,10 @@ int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = tru
   if (!pointers) return PKH3_OK;
   int rc;
   if ((rc = check_tensor("q", a->q, a->q_sb, a->q_ss, a->q_sh, a->B, a->H))) return rc;
-  if ((rc = check_tensor("k", a->k, a->k_sb, a->k_ss, a->k_sh, a->B, a->H))) return rc;
-  if ((rc = check_tensor("v", a->v, a->v_sb, a->v_ss, a->v_sh, a->B, a->H))) return rc;
+  if (need_kv && !(a->flags & PKH3_FLAG_KV_PREPARED)) {
+    if ((rc = check_tensor("k", a->k, a->k_sb, a->k_ss, a->k_sh, a->B, a->H))) return rc;
+    if ((rc = check_tensor("v", a->v, a->v_sb, a->v_ss, a->v_sh, a->B, a->H))) return rc;
+  }
   if ((rc = check_tensor("o", a->o, a->o_sb, a->o_ss, a->o_sh, a->B, a->H))) return rc;
   if (a->rope_mode != PKH3_ROPE_NONE) {
     if (!a->q_rope_cos || !a->q_rope_sin || !a->k_rope_cos || !a->k_rope_sin)
@@ -169,9 +174,46 @@ int run_prologue(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
                                 5 * L.w.nKt, (int*)(ws + L.w.plan_cnt_off), st)) != hipSuccess)
       return hip_fail(e, "sparse plan");
   }
+  if (a->flags & PKH3_FLAG_KV_PREPARED) return PKH3_OK;  // pkh3_qkv_proj wrote K, V, the scales and the row-norm maxima
   // V first: it also clears the per-head slots the K pass max-reduces its row norms into
   if ((e = launch_v_prologue(L.vp, st)) != hipSuccess) return hip_fail(e, "v prologue");
   if ((e = launch_qk_prologue(L.kp, st)) != hipSuccess) return hip_fail(e, "k prologue");
+  return PKH3_OK;
+}
+
+// ---- helpers of the projection entry points
+size_t padded_rows(int32_t rows) { return ((size_t)rows + 255) / 256 * 256; }
+
+int check_pack(const char* what, const void* x, int64_t row_stride, int32_t rows, int32_t K, const void* out) {
+  if (!x || !out) return fail(PKH3_ENULL, "%s: NULL pointer", what);
+  if (misaligned16(x)) return fail(PKH3_EALIGN, "%s: source is not 16-byte aligned", what);
+  if ((uintptr_t)out & 255u) return fail(PKH3_EALIGN, "%s: destination is not 256-byte aligned", what);
+  if (rows < 1) return fail(PKH3_ESHAPE, "%s: rows must be >= 1", what);
+  if (K < 32 || (K % 32) || K > 4096) return fail(PKH3_ESHAPE, "%s: K must be a multiple of 32 in [32, 4096], got %d", what, K);
+  if (row_stride < K || (row_stride % 8)) return fail(PKH3_ESTRIDE, "%s: row_stride must be >= K and a multiple of 8 elements", what);
+  return PKH3_OK;
+}
+
+int run_pack(const void* x, int64_t row_stride, int32_t rows, int32_t K, int head_perm, int norm, float eps, const void* shift,
+             const void* scale, int64_t table_stride, const int32_t* row_index, void* out, void* stream) {
+  PackParams p{};
+  p.x = x; p.row_stride = row_stride; p.rows = rows; p.rows_padded = (int)padded_rows(rows); p.K = K;
+  p.head_perm = head_perm; p.norm = norm; p.eps = eps; p.shift = shift; p.scale = scale; p.table_stride = table_stride;
+  p.row_index = row_index; p.out = (char*)out; p.out_blk_stride = (int64_t)(K / 16) * 1024;
+  hipError_t e = launch_pack_rows(p, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "pack_rows");
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
+int check_linear(const char* name, const pkh3_linear* l) {
+  if (!l->w_img || misaligned16(l->w_img)) return fail(PKH3_ENULL, "%s: w_img is NULL or misaligned", name);
+  if (l->bias && misaligned16(l->bias)) return fail(PKH3_EALIGN, "%s: bias is not 16-byte aligned", name);
+  if ((l->lora_a_img == nullptr) != (l->lora_b_img == nullptr))
+    return fail(PKH3_ENULL, "%s: lora_a_img and lora_b_img must be given together", name);
+  if (l->lora_a_img && (misaligned16(l->lora_a_img) || misaligned16(l->lora_b_img)))
+    return fail(PKH3_EALIGN, "%s: adapter images are not 16-byte aligned", name);
+  if (l->lora_a_img && !(l->lora_scale == l->lora_scale)) return fail(PKH3_EARG, "%s: lora_scale is not a number", name);
   return PKH3_OK;
 }
 
@@ -248,6 +290,8 @@ int pkh3_attn_fwd(const pkh3_attn_args* a, void* stream) {
 int pkh3_attn_fwd_noalloc(const pkh3_attn_args* a, void* stream) {
   int rc = validate(a, true, /*caller_workspace=*/false);
   if (rc) return rc;
+  if (a->flags & PKH3_FLAG_KV_PREPARED)
+    return fail(PKH3_EUNSUPPORTED, "pkh3_attn_fwd_noalloc: prepared K/V live in a caller workspace, which this call does not take");
   const size_t need = plan(a).total;
   if (need > (size_t)PKH3_NOALLOC_SCRATCH_BYTES)
     return fail(PKH3_EWORKSPACE,
@@ -312,6 +356,181 @@ int pkh3_rope_tables(const double* position_ids, int32_t S, const int32_t axis_d
   if (!(theta > 1.0)) return fail(PKH3_EARG, "rope_tables: theta must be > 1");
   hipError_t e = launch_rope_tables(position_ids, S, axis_dims, theta, cos_out, sin_out, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "rope_tables");
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
+// ---- projections ------------------------------------------------------------------------------------------
+
+size_t pkh3_packed_bytes(int32_t rows, int32_t K) {
+  if (rows < 1 || K < 32 || (K % 32) || K > 4096) return 0;
+  return padded_rows(rows) * (size_t)K * 2;
+}
+
+int pkh3_pack_weight(const void* w, int64_t row_stride, int32_t N, int32_t K, int32_t head_perm, void* out, void* stream) {
+  int rc = check_pack("pack_weight", w, row_stride, N, K, out);
+  if (rc) return rc;
+  if (N % 128) return fail(PKH3_ESHAPE, "pack_weight: N must be a multiple of 128 (whole heads), got %d", N);
+  return run_pack(w, row_stride, N, K, head_perm ? 1 : 0, kNormNone, 0.f, nullptr, nullptr, 0, nullptr, out, stream);
+}
+
+int pkh3_pack_rows(const void* x, int64_t row_stride, int32_t S, int32_t K, void* out, void* stream) {
+  int rc = check_pack("pack_rows", x, row_stride, S, K, out);
+  if (rc) return rc;
+  return run_pack(x, row_stride, S, K, 0, kNormNone, 0.f, nullptr, nullptr, 0, nullptr, out, stream);
+}
+
+int pkh3_adaln_modulate(const void* x, int64_t row_stride, int32_t S, int32_t K, int32_t norm_kind, float eps,
+                        const void* shift, const void* scale, int64_t table_stride, const int32_t* row_index, void* out,
+                        void* stream) {
+  int rc = check_pack("adaln_modulate", x, row_stride, S, K, out);
+  if (rc) return rc;
+  if (norm_kind < PKH3_NORM_NONE || norm_kind > PKH3_NORM_RMS) return fail(PKH3_EARG, "adaln_modulate: bad norm_kind %d", norm_kind);
+  if (norm_kind != PKH3_NORM_NONE && !(eps >= 0.f)) return fail(PKH3_EARG, "adaln_modulate: eps must be >= 0");
+  if (norm_kind == PKH3_NORM_NONE && (shift || scale))
+    return fail(PKH3_EUNSUPPORTED, "adaln_modulate: shift/scale without a norm is not implemented");
+  if ((shift && misaligned16(shift)) || (scale && misaligned16(scale)))
+    return fail(PKH3_EALIGN, "adaln_modulate: shift/scale tables must be 16-byte aligned");
+  if ((shift || scale) && (table_stride < K || (table_stride % 8)))
+    return fail(PKH3_ESTRIDE, "adaln_modulate: table_stride must be >= K and a multiple of 8 elements");
+  return run_pack(x, row_stride, S, K, 0, norm_kind, eps, shift, scale, table_stride, row_index, out, stream);
+}
+
+int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream) {
+  if (!p) return fail(PKH3_ENULL, "qkv_proj: args is NULL");
+  int rc = validate(a, true, true, /*need_kv=*/false);
+  if (rc) return rc;
+  if (a->B != 1 || a->Sq != a->Sk || a->key_mask)
+    return fail(PKH3_EUNSUPPORTED, "qkv_proj: one self-attention document only (B = 1, Sq = Sk, no key mask)");
+  if (p->S != a->Sq) return fail(PKH3_ESHAPE, "qkv_proj: S = %d but the attention call has Sq = %d", p->S, a->Sq);
+  if (p->K < 32 || (p->K % 32) || p->K > 4096) return fail(PKH3_ESHAPE, "qkv_proj: K must be a multiple of 32 in [32, 4096], got %d", p->K);
+  if (!p->x_img || misaligned16(p->x_img)) return fail(PKH3_ENULL, "qkv_proj: x_img is NULL or misaligned");
+  const pkh3_linear* lin[3] = {&p->q, &p->k, &p->v};
+  const char* names[3] = {"q", "k", "v"};
+  bool any_lora = false;
+  for (int t = 0; t < 3; ++t) {
+    if ((rc = check_linear(names[t], lin[t]))) return rc;
+    any_lora |= lin[t]->lora_a_img != nullptr;
+  }
+  const size_t lora_need = any_lora ? pkh3_packed_bytes(p->S, 3 * PKH3_LORA_RANK) : 0;
+  if (any_lora && (!p->lora_workspace || ((uintptr_t)p->lora_workspace & 255u) || p->lora_workspace_bytes < lora_need))
+    return fail(PKH3_EWORKSPACE, "qkv_proj: lora_workspace missing, misaligned (256 B) or smaller than %zu bytes", lora_need);
+  Launch L;
+  build(a, a->workspace, L);
+  if (a->workspace_bytes < L.w.total)
+    return fail(PKH3_EWORKSPACE, "workspace too small: %zu < %zu bytes", a->workspace_bytes, L.w.total);
+  hipStream_t st = (hipStream_t)stream;
+  hipError_t e;
+  const int H = a->H, N = H * kD;
+  const bool fp8 = a->flags & PKH3_FLAG_FP8_QK;
+  const int64_t w_blk = (int64_t)(p->K / 16) * 1024;       // bytes of one 32-row block of images over K
+  const int64_t b_blk = (int64_t)(PKH3_LORA_RANK / 16) * 1024;
+  const int64_t xa_blk = 3 * b_blk;                        // down-projected rows: three targets side by side
+  const int m_tiles = (int)(padded_rows(p->S) / 256);
+
+  // the K epilogue max-reduces its row norms into per-head slots that must start at zero
+  if ((e = launch_fill_zero((unsigned*)(L.ws + L.w.kmax_off), H, st)) != hipSuccess) return hip_fail(e, "fill_zero");
+
+  if (any_lora) {
+    // x A^T for the three adapters, scaled, as the activation images of the second K segment
+    GemmParams g{};
+    g.a_img = (const char*)p->x_img; g.a_blk_stride = w_blk; g.nk1 = p->K / 32; g.M = p->S; g.m_tiles = m_tiles;
+    for (int t = 0; t < 3; ++t) {
+      if (!lin[t]->lora_a_img) continue;
+      GemmTarget& tg = g.tg[g.n_targets++];
+      tg = GemmTarget{};
+      tg.epi = kEpiKImg; tg.n = PKH3_LORA_RANK; tg.n_tiles = 1;
+      tg.w_img = (const char*)lin[t]->lora_a_img; tg.w_blk_stride = w_blk;
+      tg.out_scale = lin[t]->lora_scale;
+      tg.out = (char*)p->lora_workspace + t * b_blk; tg.out_head_stride = 0;
+      tg.out_blk_stride = 2 * xa_blk; tg.out_sub_stride = (int)xa_blk;
+      tg.rope_mode = PKH3_ROPE_NONE;
+      g.n_tiles += 1;
+    }
+    if ((e = launch_gemm(g, st)) != hipSuccess) return hip_fail(e, "lora down-projection");
+  }
+
+  GemmParams g{};
+  g.a_img = (const char*)p->x_img; g.a_blk_stride = w_blk; g.nk1 = p->K / 32; g.M = p->S; g.m_tiles = m_tiles;
+  g.n_targets = 3;
+  for (int t = 0; t < 3; ++t) {
+    GemmTarget& tg = g.tg[t];
+    tg = GemmTarget{};
+    tg.n = N; tg.n_tiles = (N + 255) / 256;
+    tg.w_img = (const char*)lin[t]->w_img; tg.w_blk_stride = w_blk;
+    tg.bias = lin[t]->bias; tg.out_scale = 1.0f;
+    if (lin[t]->lora_a_img) {
+      tg.a2_img = (const char*)p->lora_workspace + t * b_blk; tg.a2_blk_stride = xa_blk;
+      tg.w2_img = (const char*)lin[t]->lora_b_img; tg.w2_blk_stride = b_blk; tg.nk2 = PKH3_LORA_RANK / 32;
+    }
+    g.n_tiles += tg.n_tiles;
+  }
+  {
+    GemmTarget& q = g.tg[0];
+    q.epi = kEpiRows; q.out = (char*)a->q; q.out_row_stride = a->q_ss; q.out_head_elems = (int)a->q_sh;
+    GemmTarget& k = g.tg[1];
+    k.epi = kEpiKImg; k.out = L.kp.out; k.out_head_stride = L.kp.out_bh_stride; k.out_blk_stride = L.kp.out_blk_stride;
+    k.out_sub_stride = fp8 ? kK8TileBytes / 2 : kKTileBytes / 2;
+    k.norm_w = a->k_norm_w; k.norm_eps = a->norm_eps; k.rope_mode = a->rope_mode; k.cos_t = a->k_rope_cos; k.sin_t = a->k_rope_sin;
+    k.norm_max = L.kp.norm_max; k.fp8 = fp8; k.scale_out = L.kp.scale_out; k.scale_head_stride = L.w.nKt;
+    GemmTarget& v = g.tg[2];
+    v.epi = kEpiVImg; v.out = L.vp.out; v.out_head_stride = L.vp.out_bh_stride; v.out_blk_stride = L.vp.out_tile_stride;
+  }
+  if (a->q_sh > INT32_MAX) return fail(PKH3_ESTRIDE, "qkv_proj: q head stride too large");
+  if ((e = launch_gemm(g, st)) != hipSuccess) return hip_fail(e, "qkv projection");
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
+int pkh3_out_proj(const pkh3_out_args* p, void* stream) {
+  if (!p) return fail(PKH3_ENULL, "out_proj: args is NULL");
+  if (p->S < 1) return fail(PKH3_ESHAPE, "out_proj: S must be >= 1");
+  if (p->K < 32 || (p->K % 32) || p->K > 4096) return fail(PKH3_ESHAPE, "out_proj: K must be a multiple of 32 in [32, 4096], got %d", p->K);
+  if (p->N < 128 || (p->N % 128)) return fail(PKH3_ESHAPE, "out_proj: N must be a multiple of 128, got %d", p->N);
+  if (!p->o_img || misaligned16(p->o_img)) return fail(PKH3_ENULL, "out_proj: o_img is NULL or misaligned");
+  if (!p->y || misaligned16(p->y)) return fail(PKH3_ENULL, "out_proj: y is NULL or misaligned");
+  if (p->y_stride < p->N || (p->y_stride % 8)) return fail(PKH3_ESTRIDE, "out_proj: y_stride must be >= N and a multiple of 8 elements");
+  if (p->gate && (misaligned16(p->gate) || p->gate_stride < p->N || (p->gate_stride % 8)))
+    return fail(PKH3_ESTRIDE, "out_proj: gate table misaligned or gate_stride not >= N and a multiple of 8");
+  if (p->residual && (misaligned16(p->residual) || p->residual_stride < p->N || (p->residual_stride % 8)))
+    return fail(PKH3_ESTRIDE, "out_proj: residual misaligned or residual_stride not >= N and a multiple of 8");
+  int rc = check_linear("to_out", &p->proj);
+  if (rc) return rc;
+  const bool lora = p->proj.lora_a_img != nullptr;
+  const size_t lora_need = lora ? pkh3_packed_bytes(p->S, PKH3_LORA_RANK) : 0;
+  if (lora && (!p->lora_workspace || ((uintptr_t)p->lora_workspace & 255u) || p->lora_workspace_bytes < lora_need))
+    return fail(PKH3_EWORKSPACE, "out_proj: lora_workspace missing, misaligned (256 B) or smaller than %zu bytes", lora_need);
+  hipStream_t st = (hipStream_t)stream;
+  hipError_t e;
+  const int64_t w_blk = (int64_t)(p->K / 16) * 1024;
+  const int64_t b_blk = (int64_t)(PKH3_LORA_RANK / 16) * 1024;
+  const int m_tiles = (int)(padded_rows(p->S) / 256);
+  if (lora) {
+    GemmParams g{};
+    g.a_img = (const char*)p->o_img; g.a_blk_stride = w_blk; g.nk1 = p->K / 32; g.M = p->S; g.m_tiles = m_tiles;
+    g.n_targets = 1; g.n_tiles = 1;
+    GemmTarget& tg = g.tg[0];
+    tg = GemmTarget{};
+    tg.epi = kEpiKImg; tg.n = PKH3_LORA_RANK; tg.n_tiles = 1;
+    tg.w_img = (const char*)p->proj.lora_a_img; tg.w_blk_stride = w_blk; tg.out_scale = p->proj.lora_scale;
+    tg.out = (char*)p->lora_workspace; tg.out_blk_stride = 2 * b_blk; tg.out_sub_stride = (int)b_blk;
+    if ((e = launch_gemm(g, st)) != hipSuccess) return hip_fail(e, "lora down-projection");
+  }
+  GemmParams g{};
+  g.a_img = (const char*)p->o_img; g.a_blk_stride = w_blk; g.nk1 = p->K / 32; g.M = p->S; g.m_tiles = m_tiles;
+  g.n_targets = 1;
+  GemmTarget& tg = g.tg[0];
+  tg = GemmTarget{};
+  tg.epi = kEpiRows; tg.n = p->N; tg.n_tiles = (p->N + 255) / 256; g.n_tiles = tg.n_tiles;
+  tg.w_img = (const char*)p->proj.w_img; tg.w_blk_stride = w_blk; tg.bias = p->proj.bias; tg.out_scale = 1.0f;
+  if (lora) {
+    tg.a2_img = (const char*)p->lora_workspace; tg.a2_blk_stride = b_blk;
+    tg.w2_img = (const char*)p->proj.lora_b_img; tg.w2_blk_stride = b_blk; tg.nk2 = PKH3_LORA_RANK / 32;
+  }
+  tg.out = (char*)p->y; tg.out_row_stride = p->y_stride; tg.out_head_elems = kD;
+  tg.gate = p->gate; tg.gate_row_stride = p->gate_stride; tg.row_index = p->row_index;
+  tg.residual = p->residual; tg.res_row_stride = p->residual_stride;
+  if ((e = launch_gemm(g, st)) != hipSuccess) return hip_fail(e, "output projection");
   g_err[0] = 0;
   return PKH3_OK;
 }

@@ -76,6 +76,81 @@ struct FwdParams {
   int unit0, units;     // filled per launch: the workgroup units [unit0, unit0 + units) this launch covers
 };
 
+// ---- projection GEMMs (pkh3_gemm.hip) -------------------------------------------------------------------
+enum { kEpiRows = 0, kEpiKImg = 1, kEpiVImg = 2 };       // what a target's epilogue writes
+enum { kNormNone = 0, kNormLayer = 1, kNormRms = 2 };    // row normalisation of the pack / modulation pass
+
+// One output of a GEMM launch: a run of `n` features (whole 128-feature heads) with its own weights and epilogue.
+struct GemmTarget {
+  int epi;                 // kEpi*
+  int n;                   // features of this target (multiple of 128)
+  int n_tiles;             // 256-feature workgroup tiles: ceil(n / 256)
+  const char* w_img;       // packed weights [feature block][k-step], head-permuted rows unless epi == kEpiVImg
+  int64_t w_blk_stride;    // bytes between consecutive 32-feature blocks
+  const float* bias;       // [n] fp32 in original feature order, or null
+  float out_scale;         // accumulator * out_scale (+ bias)
+  // second K segment (LoRA): activations from the down-projected rows of this target, weights from B
+  const char* a2_img;
+  int64_t a2_blk_stride;
+  const char* w2_img;
+  int64_t w2_blk_stride;
+  int nk2;                 // 32-wide k-chunks of the second segment (0 = none)
+  // output
+  char* out;
+  int64_t out_head_stride; // image epilogues: bytes between heads
+  int64_t out_blk_stride;  // image epilogues: bytes between 64-token tiles
+  int out_sub_stride;      // kEpiKImg: bytes between the two 32-token halves of a tile
+  int64_t out_row_stride;  // kEpiRows: elements between token rows
+  int out_head_elems;      // kEpiRows: elements between heads
+  // kEpiKImg
+  const float* norm_w;
+  float norm_eps;
+  int rope_mode;
+  const float* cos_t;
+  const float* sin_t;
+  unsigned* norm_max;      // [heads] float bits, atomic max of the row norms, or null
+  int fp8;
+  float* scale_out;        // fp8: [heads][scale_head_stride] dequantisation scales
+  int scale_head_stride;
+  // kEpiRows: y = residual + gate[row_index[token]] * (acc * out_scale + bias)
+  const void* gate;        // bf16 [rows, gate_row_stride] or null
+  int64_t gate_row_stride;
+  const int* row_index;    // [M] or null (row 0)
+  const void* residual;    // bf16 [M, res_row_stride] or null
+  int64_t res_row_stride;
+};
+
+struct GemmParams {
+  const char* a_img;       // activations [token block][k-step]
+  int64_t a_blk_stride;    // bytes between consecutive 32-token blocks
+  int nk1;                 // 32-wide k-chunks of the first segment
+  int M;                   // tokens
+  int m_tiles, n_tiles;    // 256 x 256 workgroup tiles
+  int n_targets;
+  GemmTarget tg[3];
+};
+
+// rows (activations or weights) -> operand images, optionally normalised and modulated
+struct PackParams {
+  const void* x;           // bf16 [rows, row_stride]
+  int64_t row_stride;      // elements
+  int rows, rows_padded;   // rows that exist / image rows to write (multiple of 32; the rest is zero)
+  int K;                   // elements per row (multiple of 16, <= 4096)
+  int head_perm;
+  int norm;                // kNorm*
+  float eps;
+  const void* shift;       // bf16 [table rows, table_stride] or null
+  const void* scale;
+  int64_t table_stride;
+  const int* row_index;    // [rows] table row of each row, or null (row 0)
+  char* out;
+  int64_t out_blk_stride;  // bytes between consecutive 32-row blocks
+};
+
+hipError_t launch_gemm(const GemmParams& p, hipStream_t st);
+hipError_t launch_pack_rows(const PackParams& p, hipStream_t st);
+hipError_t launch_fill_zero(unsigned* p, int n, hipStream_t st);
+
 hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int* cnt, hipStream_t st);
 hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st);
 hipError_t launch_v_prologue(const VPrologueParams& p, hipStream_t st);

@@ -70,26 +70,33 @@ def _f32(name: str, t: Optional[torch.Tensor], shape, device) -> Optional[torch.
 def fill_args(
     q, k, v, out, *, q_norm_weight=None, k_norm_weight=None, norm_eps=1e-6, rope_q=None, rope_k=None,
     rope_mode=_lib.ROPE_NONE, key_mask=None, block_mask: Optional[BlockMask] = None, fp8_qk=False,
-    softmax_scale: Optional[float] = None, long_key_kernel: bool = False,
+    softmax_scale: Optional[float] = None, long_key_kernel: bool = False, kv_prepared: bool = False,
 ) -> Tuple[_lib.AttnArgs, list]:
-    """Build ``pkh3_attn_args`` for these tensors.  Returns (args, keep_alive)."""
+    """Build ``pkh3_attn_args`` for these tensors.  Returns (args, keep_alive).  ``kv_prepared``: K and V
+    come from the fused projection (``pkh3_qkv_proj``) through the workspace; ``k`` and ``v`` are then None."""
+    if kv_prepared != (k is None) or (k is None) != (v is None):
+        raise ValueError("k and v are None exactly when kv_prepared is set")
     for n, t in (("q", q), ("k", k), ("v", v), ("out", out)):
-        _check_bshd(n, t)
+        if t is not None:
+            _check_bshd(n, t)
     B, Sq, H, D = q.shape
-    Sk = k.shape[1]
-    if tuple(k.shape) != (B, Sk, H, D) or tuple(v.shape) != (B, Sk, H, D):
+    Sk = Sq if k is None else k.shape[1]
+    if k is not None and (tuple(k.shape) != (B, Sk, H, D) or tuple(v.shape) != (B, Sk, H, D)):
         raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
     if tuple(out.shape) != (B, Sq, H, D):
         raise ValueError(f"out shape {tuple(out.shape)} != {(B, Sq, H, D)}")
     dev = q.device
     for n, t in (("k", k), ("v", v), ("out", out)):
-        _on_device(n, t, dev)
+        if t is not None:
+            _on_device(n, t, dev)
     keep = [q, k, v, out]
     a = _lib.AttnArgs()
-    a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.q, a.o = q.data_ptr(), out.data_ptr()
     a.q_sb, a.q_ss, a.q_sh = q.stride(0), q.stride(1), q.stride(2)
-    a.k_sb, a.k_ss, a.k_sh = k.stride(0), k.stride(1), k.stride(2)
-    a.v_sb, a.v_ss, a.v_sh = v.stride(0), v.stride(1), v.stride(2)
+    if k is not None:
+        a.k, a.v = k.data_ptr(), v.data_ptr()
+        a.k_sb, a.k_ss, a.k_sh = k.stride(0), k.stride(1), k.stride(2)
+        a.v_sb, a.v_ss, a.v_sh = v.stride(0), v.stride(1), v.stride(2)
     a.o_sb, a.o_ss, a.o_sh = out.stride(0), out.stride(1), out.stride(2)
     a.B, a.H, a.Sq, a.Sk, a.D = B, H, Sq, Sk, D
     a.softmax_scale = float(softmax_scale) if softmax_scale is not None else 0.0
@@ -129,7 +136,8 @@ def fill_args(
             raise ValueError("block mask CSR arrays must be contiguous")
         a.blk_row_ptr, a.blk_col_idx = block_mask.row_ptr.data_ptr(), block_mask.col_idx.data_ptr()
         keep += [block_mask.row_ptr, block_mask.col_idx]
-    a.flags = (_lib.FLAG_FP8_QK if fp8_qk else 0) | (_lib.FLAG_LONG_KEY_KERNEL if long_key_kernel else 0)
+    a.flags = ((_lib.FLAG_FP8_QK if fp8_qk else 0) | (_lib.FLAG_LONG_KEY_KERNEL if long_key_kernel else 0)
+               | (_lib.FLAG_KV_PREPARED if kv_prepared else 0))
     keep += [qw, kw]
     return a, keep
 

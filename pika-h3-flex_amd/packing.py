@@ -121,8 +121,8 @@ class PackedLayout:
 
     position_ids: torch.Tensor   # [S, 3] float64 (t, h, w)
     token_tags: torch.Tensor     # [S] int64: 0 video, 1 text, 2 audio
-    video_indices: torch.Tensor  # rows of the target video, int64
-    audio_indices: torch.Tensor  # rows of the target audio
+    video_indices: torch.Tensor  # rows of the video modality, condition (keyframe) rows first, then the targets; int64
+    audio_indices: torch.Tensor  # rows of the audio modality, condition rows first, then the targets
     text_indices: torch.Tensor   # rows of the text
     num_condition_video_rows: int
     num_condition_audio_rows: int
@@ -182,15 +182,46 @@ def build_layout(*, num_text_tokens: int, num_latent_frames: int, latent_height:
     pos.append(video_position_ids(num_latent_frames, hp, wp))
     tags.append(torch.full((counts.video,), VIDEO_TAG, dtype=torch.int64))
     position_ids, token_tags = torch.cat(pos), torch.cat(tags)
-    a0 = counts.text + counts.condition_video + counts.condition_audio
+    cv0 = counts.text
+    ca0 = cv0 + counts.condition_video
+    a0 = ca0 + counts.condition_audio
     v0 = a0 + counts.audio
+    # the index sets list ALL rows of a modality, condition rows first: the wrapper concatenates condition and target
+    # rows per modality and checks the totals against them (src/pika_h3/core/wrapper.py:171-179)
     return PackedLayout(
         position_ids=position_ids, token_tags=token_tags,
-        video_indices=torch.arange(v0, v0 + counts.video, dtype=torch.int64),
-        audio_indices=torch.arange(a0, a0 + counts.audio, dtype=torch.int64),
+        video_indices=torch.cat([torch.arange(cv0, cv0 + counts.condition_video, dtype=torch.int64),
+                                 torch.arange(v0, v0 + counts.video, dtype=torch.int64)]),
+        audio_indices=torch.arange(ca0, a0 + counts.audio, dtype=torch.int64),
         text_indices=torch.arange(0, counts.text, dtype=torch.int64),
         num_condition_video_rows=counts.condition_video, num_condition_audio_rows=counts.condition_audio,
         num_text_tokens=counts.text, counts=counts)
+
+
+def row_timesteps(layout: PackedLayout, *, video_t: float, audio_t: float, condition_video_t: float,
+                  condition_audio_t: float = 1.0, text_t: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(unique timesteps ``[K]`` float32 ascending, per-row index ``[S]`` int32 into them): the ``timestep`` /
+    ``timestep_indices`` pair of the model call (src/pika_h3/core/wrapper.py:182-190,196-197), by which every
+    block gathers its AdaLN parameters per row (patches/0001-h3-adaln-fp32.patch:39-40).
+
+    Argument list as in src/pika_h3/core/packing.py:212-231: target video rows sit at ``video_t``, target audio
+    rows at ``audio_t``, condition rows at their pinned times (the wrapper passes ``max(video_t, noise_aug)``
+    and 1.0, clean-time convention).  The rule itself lives in the reference's un-vendored diffusers pin
+    (``build_row_timesteps``); what that file alone fixes is a switch here: text rows take ``text_t`` (clean by
+    default) and the unique values are listed in ascending order.
+    """
+    S = layout.sequence_length
+    t = torch.full((S,), float(text_t), dtype=torch.float64)
+    n_cv, n_ca = layout.num_condition_video_rows, layout.num_condition_audio_rows
+    vi, ai = layout.video_indices.cpu(), layout.audio_indices.cpu()
+    t[vi[:n_cv]] = float(condition_video_t)
+    t[vi[n_cv:]] = float(video_t)
+    t[ai[:n_ca]] = float(condition_audio_t)
+    t[ai[n_ca:]] = float(audio_t)
+    if layout.num_text_tokens == 0 and vi.numel() + ai.numel() != S:
+        raise ValueError("layout rows are not covered by its index sets")
+    unique, index = torch.unique(t, sorted=True, return_inverse=True)
+    return unique.to(torch.float32), index.to(torch.int32)
 
 
 class LayoutCache:

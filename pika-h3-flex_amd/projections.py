@@ -1,0 +1,231 @@
+"""Tensor-level front end of the projection entry points of the C ABI: the ``to_q / to_k / to_v /
+to_out.0`` linear layers of the attention module with their LoRA adapters (target list
+src/pika_h3/core/loader.py:9, injection src/pika_h3/core/loader.py:20-49) and the AdaLN modulation
+that feeds them (patches/0001-h3-adaln-fp32.patch:34-40).  PyTorch supplies device memory and the
+stream; all arithmetic happens in libpkh3attn.so.
+
+Matrix operands live in "operand images" (uint8 tensors here): weights are packed once with
+:func:`pack_weight` / :meth:`PackedLinear.from_weights`, activations by :func:`adaln_modulate` or
+:func:`pack_rows`.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .ops import HEAD_DIM, _on_device, fill_args, workspace_bytes
+
+NORMS = {"none": _lib.NORM_NONE, "layer": _lib.NORM_LAYER, "rms": _lib.NORM_RMS}
+
+
+def _stream(device) -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _rows_bf16(name: str, t: torch.Tensor) -> torch.Tensor:
+    if t.dim() != 2 or t.dtype != torch.bfloat16 or t.stride(1) != 1:
+        raise ValueError(f"{name} must be a bfloat16 [rows, K] matrix with unit column stride, got {t.dtype} {tuple(t.shape)}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live in device memory (got {t.device}); the HIP library is the only compute path")
+    return t
+
+
+def packed_bytes(rows: int, K: int) -> int:
+    n = _lib.load().pkh3_packed_bytes(int(rows), int(K))
+    if n == 0:
+        raise ValueError(f"cannot pack a [{rows}, {K}] matrix: K must be a multiple of 32 in [32, 4096]")
+    return int(n)
+
+
+def pack_weight(w: torch.Tensor, *, head_perm: bool = True) -> torch.Tensor:
+    """``w`` bf16 ``[N, K]`` (``torch.nn.Linear.weight``) -> operand images.  ``head_perm=False`` for a V
+    projection (and the LoRA B that goes with it)."""
+    w = _rows_bf16("weight", w)
+    N, K = w.shape
+    out = torch.empty(packed_bytes(N, K), dtype=torch.uint8, device=w.device)
+    with torch.cuda.device(w.device):
+        _lib.check(_lib.load().pkh3_pack_weight(w.data_ptr(), w.stride(0), N, K, int(head_perm), out.data_ptr(), _stream(w.device)))
+    return out
+
+
+def pack_rows(x: torch.Tensor) -> torch.Tensor:
+    """Activations bf16 ``[S, K]`` -> operand images."""
+    x = _rows_bf16("x", x)
+    S, K = x.shape
+    out = torch.empty(packed_bytes(S, K), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().pkh3_pack_rows(x.data_ptr(), x.stride(0), S, K, out.data_ptr(), _stream(x.device)))
+    return out
+
+
+def adaln_modulate(x: torch.Tensor, *, shift: Optional[torch.Tensor] = None, scale: Optional[torch.Tensor] = None,
+                   row_index: Optional[torch.Tensor] = None, norm: str = "layer", eps: float = 1e-6) -> torch.Tensor:
+    """``norm(x) * (1 + scale[row_index]) + shift[row_index]`` for ``x`` bf16 ``[S, K]``, as operand images.
+    ``shift`` / ``scale``: bf16 ``[table rows, K]``; ``row_index`` int32 ``[S]`` (None: table row 0)."""
+    x = _rows_bf16("x", x)
+    S, K = x.shape
+    stride = 0
+    for name, t in (("shift", shift), ("scale", scale)):
+        if t is None:
+            continue
+        _rows_bf16(name, t)
+        _on_device(name, t, x.device)
+        if t.shape[1] != K:
+            raise ValueError(f"{name} must have {K} columns, got {t.shape[1]}")
+        if stride and t.stride(0) != stride:
+            raise ValueError("shift and scale must share one row stride")
+        stride = t.stride(0)
+    if shift is not None and scale is not None and shift.shape[0] != scale.shape[0]:
+        raise ValueError("shift and scale must have the same number of rows")
+    if row_index is not None:
+        if row_index.dtype != torch.int32 or tuple(row_index.shape) != (S,) or not row_index.is_contiguous():
+            raise ValueError(f"row_index must be contiguous int32 [{S}]")
+        _on_device("row_index", row_index, x.device)
+    out = torch.empty(packed_bytes(S, K), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().pkh3_adaln_modulate(
+            x.data_ptr(), x.stride(0), S, K, NORMS[norm], float(eps),
+            None if shift is None else shift.data_ptr(), None if scale is None else scale.data_ptr(), stride,
+            None if row_index is None else row_index.data_ptr(), out.data_ptr(), _stream(x.device)))
+    return out
+
+
+@dataclass
+class PackedLinear:
+    """One linear layer, packed: ``y = x W^T + bias + lora_scale * (x A^T) B^T``."""
+
+    w_img: torch.Tensor
+    N: int
+    K: int
+    bias: Optional[torch.Tensor] = None        # fp32 [N]
+    lora_a_img: Optional[torch.Tensor] = None
+    lora_b_img: Optional[torch.Tensor] = None
+    lora_scale: float = 0.0
+
+    @staticmethod
+    def from_weights(weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *, lora_a: Optional[torch.Tensor] = None,
+                     lora_b: Optional[torch.Tensor] = None, lora_scale: float = 1.0, head_perm: bool = True) -> "PackedLinear":
+        """``weight [N, K]``, ``lora_a [rank, K]``, ``lora_b [N, rank]`` in bf16 on the device; rank must be 128."""
+        N, K = weight.shape
+        pl = PackedLinear(pack_weight(weight, head_perm=head_perm), int(N), int(K))
+        if bias is not None:
+            pl.bias = bias.detach().to(device=weight.device, dtype=torch.float32).contiguous()
+        if (lora_a is None) != (lora_b is None):
+            raise ValueError("lora_a and lora_b go together")
+        if lora_a is not None:
+            if tuple(lora_a.shape) != (_lib.LORA_RANK, K) or tuple(lora_b.shape) != (N, _lib.LORA_RANK):
+                raise ValueError(f"adapter shapes must be A [{_lib.LORA_RANK}, {K}] and B [{N}, {_lib.LORA_RANK}], got "
+                                 f"{tuple(lora_a.shape)} and {tuple(lora_b.shape)}")
+            pl.lora_a_img = pack_weight(lora_a.to(torch.bfloat16), head_perm=True)
+            pl.lora_b_img = pack_weight(lora_b.to(torch.bfloat16), head_perm=head_perm)
+            pl.lora_scale = float(lora_scale)
+        return pl
+
+    @staticmethod
+    def from_module(mod, *, head_perm: bool = True, adapter: str = "default") -> "PackedLinear":
+        """From a ``torch.nn.Linear`` or a PEFT-style LoRA wrapper around one (``base_layer``, ``lora_A[adapter]``,
+        ``lora_B[adapter]``, ``scaling[adapter]``: what ``add_adapter`` leaves on the targets of
+        src/pika_h3/core/loader.py:36-37)."""
+        base = getattr(mod, "base_layer", mod)
+        kw = {}
+        if hasattr(mod, "lora_A") and adapter in mod.lora_A:
+            kw = dict(lora_a=mod.lora_A[adapter].weight.detach(), lora_b=mod.lora_B[adapter].weight.detach(),
+                      lora_scale=float(mod.scaling[adapter]))
+        return PackedLinear.from_weights(base.weight.detach().to(torch.bfloat16), getattr(base, "bias", None),
+                                         head_perm=head_perm, **kw)
+
+    def c_struct(self) -> _lib.Linear:
+        s = _lib.Linear()
+        s.w_img = self.w_img.data_ptr()
+        s.bias = None if self.bias is None else self.bias.data_ptr()
+        s.lora_a_img = None if self.lora_a_img is None else self.lora_a_img.data_ptr()
+        s.lora_b_img = None if self.lora_b_img is None else self.lora_b_img.data_ptr()
+        s.lora_scale = self.lora_scale
+        return s
+
+
+def qkv_attention(x_img: torch.Tensor, S: int, q: PackedLinear, k: PackedLinear, v: PackedLinear, *, heads: int,
+                  out: Optional[torch.Tensor] = None, return_q: bool = False, **opts) -> torch.Tensor:
+    """One self-attention call from packed activations: ``to_q / to_k / to_v`` (+ adapters) with the K side's
+    norm + rotation (+ fp8 quantisation) and the K/V layout in the GEMM epilogue, then the attention kernel on
+    what the GEMM left in the workspace.  ``opts`` are those of :func:`ops.fill_args` (norm weights, rope
+    tables, ``fp8_qk``, ``block_mask`` ...).  Returns O ``[1, S, H, D]`` bf16 (and Q when ``return_q``)."""
+    lib = _lib.load()
+    dev = x_img.device
+    K = q.K
+    for name, pl in (("q", q), ("k", k), ("v", v)):
+        if pl.N != heads * HEAD_DIM or pl.K != K:
+            raise ValueError(f"{name} projection is [{pl.N}, {pl.K}], expected [{heads * HEAD_DIM}, {K}]")
+    if x_img.dtype != torch.uint8 or x_img.numel() < packed_bytes(S, K):
+        raise ValueError("x_img is not a packed [S, K] activation buffer")
+    qt = torch.empty((1, S, heads, HEAD_DIM), dtype=torch.bfloat16, device=dev)
+    if out is None:
+        out = torch.empty_like(qt)
+    args, keep = fill_args(qt, None, None, out, kv_prepared=True, **opts)
+    ws = torch.empty(workspace_bytes(args), dtype=torch.uint8, device=dev)
+    args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+    pa = _lib.QkvArgs()
+    pa.x_img, pa.S, pa.K = x_img.data_ptr(), int(S), int(K)
+    pa.q, pa.k, pa.v = q.c_struct(), k.c_struct(), v.c_struct()
+    lws = None
+    if any(pl.lora_a_img is not None for pl in (q, k, v)):
+        lws = torch.empty(packed_bytes(S, 3 * _lib.LORA_RANK), dtype=torch.uint8, device=dev)
+        pa.lora_workspace, pa.lora_workspace_bytes = lws.data_ptr(), lws.numel()
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream()
+        _lib.check(lib.pkh3_qkv_proj(C.byref(pa), C.byref(args), C.c_void_p(stream.cuda_stream)))
+        _lib.check(lib.pkh3_attn_fwd(C.byref(args), C.c_void_p(stream.cuda_stream)))
+        ws.record_stream(stream)
+        if lws is not None:
+            lws.record_stream(stream)
+    return (out, qt) if return_q else out
+
+
+def out_proj(o: torch.Tensor, proj: PackedLinear, *, gate: Optional[torch.Tensor] = None,
+             row_index: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``residual + gate[row_index] * (o W^T + bias + adapter)`` for the attention output ``o`` bf16 ``[S, K]``
+    (e.g. ``O.view(S, H*D)``).  ``gate`` bf16 ``[table rows, N]``, ``residual`` bf16 ``[S, N]``."""
+    lib = _lib.load()
+    o = _rows_bf16("o", o)
+    S, K = o.shape
+    if K != proj.K:
+        raise ValueError(f"o has {K} columns, the projection expects {proj.K}")
+    dev = o.device
+    o_img = pack_rows(o)
+    y = torch.empty((S, proj.N), dtype=torch.bfloat16, device=dev)
+    a = _lib.OutArgs()
+    a.o_img, a.S, a.K, a.N = o_img.data_ptr(), S, K, proj.N
+    a.proj = proj.c_struct()
+    if gate is not None:
+        _rows_bf16("gate", gate)
+        _on_device("gate", gate, dev)
+        if gate.shape[1] != proj.N:
+            raise ValueError(f"gate must have {proj.N} columns")
+        a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
+        if row_index is not None:
+            if row_index.dtype != torch.int32 or tuple(row_index.shape) != (S,) or not row_index.is_contiguous():
+                raise ValueError(f"row_index must be contiguous int32 [{S}]")
+            _on_device("row_index", row_index, dev)
+            a.row_index = row_index.data_ptr()
+    if residual is not None:
+        _rows_bf16("residual", residual)
+        _on_device("residual", residual, dev)
+        if tuple(residual.shape) != (S, proj.N):
+            raise ValueError(f"residual must be [{S}, {proj.N}]")
+        a.residual, a.residual_stride = residual.data_ptr(), residual.stride(0)
+    a.y, a.y_stride = y.data_ptr(), y.stride(0)
+    lws = None
+    if proj.lora_a_img is not None:
+        lws = torch.empty(packed_bytes(S, _lib.LORA_RANK), dtype=torch.uint8, device=dev)
+        a.lora_workspace, a.lora_workspace_bytes = lws.data_ptr(), lws.numel()
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream()
+        _lib.check(lib.pkh3_out_proj(C.byref(a), C.c_void_p(stream.cuda_stream)))
+        o_img.record_stream(stream)
+        if lws is not None:
+            lws.record_stream(stream)
+    return y

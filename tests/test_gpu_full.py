@@ -390,9 +390,9 @@ def test_processor_on_a_packed_document():
     # per-modality input embeddings (random stand-ins for the model's patch embedders), scattered by the index sets
     x = torch.zeros(1, S, hidden)
     x[0, lay.text_indices] = torch.randn(n_text, hidden)
-    x[0, n_text:n_text + key_rows.shape[1]] = key_rows[0] @ torch.randn(96, hidden) * 0.1
+    # condition (keyframe) rows come first in the video index set, as the wrapper concatenates them
     x[0, lay.audio_indices] = audio_rows[0] @ torch.randn(32, hidden) * 0.2
-    x[0, lay.video_indices] = video_rows[0] @ torch.randn(96, hidden) * 0.1
+    x[0, lay.video_indices] = torch.cat([key_rows[0], video_rows[0]]) @ torch.randn(96, hidden) * 0.1
     x = x.cuda().to(torch.bfloat16)
     attn = _Attn(hidden, H).cuda().to(torch.bfloat16)
     proc = pk.PikaH3AttnProcessor()

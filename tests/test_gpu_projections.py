@@ -1,0 +1,215 @@
+"""GPU parity of the projection entry points (pkh3_pack_*, pkh3_adaln_modulate, pkh3_qkv_proj, pkh3_out_proj)
+against the float64 oracle (oracle/projection_oracle.py), through the C ABI.
+
+bf16 bar of the path: max-abs <= 2e-2 and cosine >= 0.9999 against float64 on tensors of unit scale; the fp8 /
+block-sparse attention variants keep their cosine >= 0.995 bar.  The operand-image layout is checked against its
+documented index formula, written out here independently of the kernels."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+D = 128
+
+
+def _r(*shape, seed=0, std=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * std
+
+
+def _unpack(buf, rows, K):
+    """Operand images -> matrix: image (rb, ks) holds rows 32*rb..+31; lane 32*hh + r carries elements
+    16*ks + 8*hh + 0..7 of row 32*rb + r."""
+    img = buf.view(torch.bfloat16).view(-1, K // 16, 2, 32, 8)      # [rb, ks, hh, r, j]
+    return img.permute(0, 3, 1, 2, 4).reshape(-1, K)[:rows]
+
+
+def _head_perm_source(rho):
+    """Source row (inside its 128-row head) of image row ``rho``: 32*db + 8*a + 4*h + b <- 32*db + 16*(a>>1) + 8*h + 4*(a&1) + b."""
+    db, q = rho // 32, rho % 32
+    a, h, b = q // 8, (q // 4) % 2, q % 4
+    return 32 * db + 16 * (a >> 1) + 8 * h + 4 * (a & 1) + b
+
+
+def test_pack_layout_matches_its_index_formula():
+    from pika_h3_flex_amd import projections as P
+
+    x = _r(70, 96, seed=1).to(torch.bfloat16).cuda()
+    buf = P.pack_rows(x)
+    assert buf.numel() == 256 * 96 * 2                                # rows padded to 256
+    torch.cuda.synchronize()
+    full = _unpack(buf, 256, 96)
+    assert torch.equal(full[:70].cpu(), x.cpu()) and float(full[70:].float().abs().sum()) == 0.0
+    # a strided source (a column slice of a wider matrix)
+    wide = _r(40, 200, seed=2).to(torch.bfloat16).cuda()
+    assert torch.equal(_unpack(P.pack_rows(wide[:, 8:104]), 40, 96).cpu(), wide[:, 8:104].cpu())
+    # weights: identity order for a V projection, permuted inside every 128-row head otherwise
+    w = _r(256, 64, seed=3).to(torch.bfloat16).cuda()
+    assert torch.equal(_unpack(P.pack_weight(w, head_perm=False), 256, 64).cpu(), w.cpu())
+    got = _unpack(P.pack_weight(w, head_perm=True), 256, 64).cpu()
+    src = torch.tensor([128 * (r // 128) + _head_perm_source(r % 128) for r in range(256)])
+    assert sorted(src.tolist()) == list(range(256))                   # a permutation
+    assert torch.equal(got, w.cpu()[src])
+
+
+@pytest.mark.parametrize("norm", ["layer", "rms"])
+def test_adaln_modulate_matches_oracle(norm):
+    from oracle import attention_oracle as AO
+    from oracle import projection_oracle as PO
+    from pika_h3_flex_amd import projections as P
+
+    S, K, T = 333, 3072, 4
+    x = (_r(S, K, seed=4) * 2 + 0.3).to(torch.bfloat16)
+    shift, scale = _r(T, K, seed=5, std=0.3).to(torch.bfloat16), _r(T, K, seed=6, std=0.3).to(torch.bfloat16)
+    idx = torch.randint(0, T, (S,), generator=torch.Generator().manual_seed(7)).to(torch.int32)
+    img = P.adaln_modulate(x.cuda(), shift=shift.cuda(), scale=scale.cuda(), row_index=idx.cuda(), norm=norm)
+    torch.cuda.synchronize()
+    got = _unpack(img, S, K).cpu()
+    ref = PO.adaln_modulate(x, shift=shift, scale=scale, row_index=idx, norm=norm)
+    err, cos = AO.max_abs_and_cosine(got, ref)
+    print(f"adaln {norm}: max_abs={err:.3e} cos={cos:.8f}", flush=True)
+    assert cos >= 0.99999 and float(((got.double() - ref).abs() / (ref.abs() + 1.0)).max()) <= 2.0 ** -8   # one bf16 rounding
+    # without tables: the bare norm; without an index: table row 0
+    bare = _unpack(P.adaln_modulate(x.cuda(), norm=norm), S, K).cpu()
+    assert AO.max_abs_and_cosine(bare, PO.adaln_modulate(x, norm=norm))[1] >= 0.99999
+    row0 = _unpack(P.adaln_modulate(x.cuda(), shift=shift.cuda(), scale=scale.cuda(), norm=norm), S, K).cpu()
+    assert AO.max_abs_and_cosine(row0, PO.adaln_modulate(x, shift=shift, scale=scale, norm=norm))[1] >= 0.99999
+
+
+def _linear(n, k, seed, lora=True, bias=True):
+    d = dict(weight=_r(n, k, seed=seed, std=k ** -0.5).to(torch.bfloat16))
+    if bias:
+        d["bias"] = _r(n, seed=seed + 1, std=0.1)
+    if lora:
+        d.update(lora_a=_r(128, k, seed=seed + 2, std=k ** -0.5).to(torch.bfloat16),
+                 lora_b=_r(n, 128, seed=seed + 3, std=0.05).to(torch.bfloat16), lora_scale=0.5)
+    return d
+
+
+def _packed(d, head_perm=True):
+    from pika_h3_flex_amd.projections import PackedLinear
+
+    return PackedLinear.from_weights(d["weight"].cuda(), d["bias"].cuda() if "bias" in d else None,
+                                     lora_a=d["lora_a"].cuda() if "lora_a" in d else None,
+                                     lora_b=d["lora_b"].cuda() if "lora_b" in d else None,
+                                     lora_scale=d.get("lora_scale", 1.0), head_perm=head_perm)
+
+
+@pytest.mark.parametrize("S,H,variant", [
+    (300, 2, "bf16"), (777, 3, "bf16"), (64, 1, "bf16"), (1000, 2, "no_lora"), (520, 2, "fp8"), (700, 2, "sparse"),
+    (450, 3, "rope_half"),
+])
+def test_qkv_projection_feeds_attention(S, H, variant):
+    """to_q/to_k/to_v (+LoRA, bias) with the K-side norm + rotation and the K/V layout in the GEMM epilogue, then the
+    attention kernel on the prepared workspace: Q against lora_linear, O against the oracle's composition."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as AO
+    from oracle import projection_oracle as PO
+    from pika_h3_flex_amd import projections as P
+
+    C = H * D
+    lora = variant != "no_lora"
+    x = _r(S, C, seed=10).to(torch.bfloat16)
+    lin = {n: _linear(C, C, 20 + 10 * i, lora=lora, bias=(n != "k")) for i, n in enumerate(("q", "k", "v"))}
+    wq, wk = 1.0 + 0.1 * _r(D, seed=50), 1.0 + 0.1 * _r(D, seed=51)
+    pos = torch.cat([pk.video_position_ids(1, 1, S - 20), pk.audio_position_ids(10)], 0)
+    mode = pk.ROPE_HALF if variant == "rope_half" else pk.ROPE_INTERLEAVED
+    opts = dict(q_norm_weight=wq.cuda(), k_norm_weight=wk.cuda(), rope_mode=mode, rope_q=pk.rope_tables(pos.cuda()))
+    ref_opts = dict(q_norm_weight=wq, k_norm_weight=wk, rope_mode=mode, rope_q=AO.rope_tables(pos))
+    if variant == "fp8":
+        opts.update(fp8_qk=True)
+        ref_opts.update(fp8_qk=True)
+    if variant == "sparse":
+        n = (S + 63) // 64
+        tm = (torch.rand((n, n), generator=torch.Generator().manual_seed(3)) < 0.5) | torch.eye(n, dtype=torch.bool)
+        opts.update(block_mask=pk.BlockMask.from_dense(tm, device="cuda"))
+        ref_opts.update(tile_map=tm)
+    out, q = P.qkv_attention(P.pack_rows(x.cuda()), S, _packed(lin["q"]), _packed(lin["k"]), _packed(lin["v"], head_perm=False),
+                             heads=H, return_q=True, **opts)
+    torch.cuda.synchronize()
+    q_ref = PO.lora_linear(x, **lin["q"]).view(1, S, H, D)
+    err, cos = AO.max_abs_and_cosine(q.cpu(), q_ref)
+    print(f"[{variant} S={S} H={H}] Q: max_abs={err:.3e} cos={cos:.8f}", flush=True)
+    assert err <= 2e-2 and cos >= 0.9999
+    # attention on bf16-rounded Q, K, V (what the product stores between its kernels; K is rounded after norm+rope
+    # inside the epilogue instead, which the bf16 bar absorbs)
+    r = lambda t: t.to(torch.bfloat16)
+    k_ref, v_ref = (PO.lora_linear(x, **lin[n]).view(1, S, H, D) for n in ("k", "v"))
+    o_ref = AO.reference_layer(r(q_ref), r(k_ref), r(v_ref), **ref_opts)
+    err, cos = AO.max_abs_and_cosine(out.cpu(), o_ref)
+    print(f"[{variant} S={S} H={H}] O: max_abs={err:.3e} cos={cos:.8f}", flush=True)
+    assert torch.isfinite(out.float()).all()
+    if variant == "fp8":
+        assert cos >= 0.995
+    else:
+        assert err <= 2e-2 and cos >= 0.9999
+    # and against the unfused route on the same Q, K, V (torch GEMM -> K/V pass -> same attention kernel)
+    unfused = pk.attention(r(q_ref).cuda(), r(k_ref).cuda(), r(v_ref).cuda(), **opts)
+    torch.cuda.synchronize()
+    err, cos = AO.max_abs_and_cosine(out.cpu(), unfused.cpu())
+    assert cos >= (0.995 if variant == "fp8" else 0.9999)
+
+
+@pytest.mark.parametrize("S,N,K,lora,extras", [(300, 256, 256, True, True), (1000, 384, 256, False, True), (65, 128, 512, True, False)])
+def test_out_projection_with_gate_and_residual(S, N, K, lora, extras):
+    from oracle import attention_oracle as AO
+    from oracle import projection_oracle as PO
+    from pika_h3_flex_amd import projections as P
+
+    o = _r(S, K, seed=60).to(torch.bfloat16)
+    lin = _linear(N, K, 61, lora=lora)
+    T = 3
+    gate = _r(T, N, seed=70, std=0.5).to(torch.bfloat16)
+    idx = torch.randint(0, T, (S,), generator=torch.Generator().manual_seed(71)).to(torch.int32)
+    res = _r(S, N, seed=72).to(torch.bfloat16)
+    kw = dict(gate=gate.cuda(), row_index=idx.cuda(), residual=res.cuda()) if extras else {}
+    y = P.out_proj(o.cuda(), _packed(lin), **kw)
+    torch.cuda.synchronize()
+    ref = PO.lora_linear(o, **lin)
+    if extras:
+        ref = res.double() + gate.double()[idx.long()] * ref
+    err, cos = AO.max_abs_and_cosine(y.cpu(), ref)
+    print(f"out_proj S={S} N={N} K={K} lora={lora}: max_abs={err:.3e} cos={cos:.8f}", flush=True)
+    assert err <= 2e-2 * max(1.0, float(ref.abs().max())) and cos >= 0.9999
+
+
+def test_attention_block_at_480p_shapes():
+    """The whole attention half of a block at the benchmark's size (S = 48,360, hidden 3072, 24 heads, LoRA rank 128 on
+    all four projections): modulate -> fused QKV -> attention -> to_out with gate and residual, against the float64
+    oracle run on the card for every row."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as AO
+    from oracle import projection_oracle as PO
+    from pika_h3_flex_amd import projections as P
+
+    S, H = 48360, 24
+    C = H * D
+    dev = "cuda"
+    x = _r(S, C, seed=80).to(torch.bfloat16).to(dev)
+    lin = {n: {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in _linear(C, C, 90 + 10 * i).items()}
+           for i, n in enumerate(("q", "k", "v", "out"))}
+    T = 3
+    shift, scale, gate = (_r(T, C, seed=s, std=0.2).to(torch.bfloat16).to(dev) for s in (130, 131, 132))
+    pos = pk.video_position_ids(31, 30, 52).to(dev)
+    idx = (torch.arange(S) * T // S).to(torch.int32).to(dev)
+    ones = torch.ones(D, device=dev)
+    x_img = P.adaln_modulate(x, shift=shift, scale=scale, row_index=idx, norm="layer")
+    packed = {n: PackedLinear_from(lin[n], head_perm=(n != "v")) for n in lin}
+    out = P.qkv_attention(x_img, S, packed["q"], packed["k"], packed["v"], heads=H, q_norm_weight=ones, k_norm_weight=ones,
+                          rope_mode=pk.ROPE_INTERLEAVED, rope_q=pk.rope_tables(pos))
+    y = P.out_proj(out.view(S, C), packed["out"], gate=gate, row_index=idx, residual=x)
+    torch.cuda.synchronize()
+    ref = PO.attention_block(x, lin, heads=H, shift=shift, scale=scale, gate=gate, row_index=idx, norm="layer",
+                             q_norm_weight=ones, k_norm_weight=ones, rope_mode=AO.ROPE_INTERLEAVED, rope_q=AO.rope_tables(pos))
+    err_o, cos_o = AO.max_abs_and_cosine(out.view(S, C), ref["o"])
+    err_y, cos_y = AO.max_abs_and_cosine(y, ref["y"])
+    print(f"480p block: O max_abs={err_o:.3e} cos={cos_o:.8f}; y max_abs={err_y:.3e} cos={cos_y:.8f}", flush=True)
+    assert torch.isfinite(y.float()).all()
+    assert err_o <= 2e-2 and cos_o >= 0.9999
+    assert err_y <= 2e-2 * max(1.0, float(ref["y"].abs().max())) and cos_y >= 0.9999
+
+
+def PackedLinear_from(d, head_perm=True):
+    from pika_h3_flex_amd.projections import PackedLinear
+
+    return PackedLinear.from_weights(d["weight"], d.get("bias"), lora_a=d.get("lora_a"), lora_b=d.get("lora_b"),
+                                     lora_scale=d.get("lora_scale", 1.0), head_perm=head_perm)

@@ -65,8 +65,13 @@ def test_layout_order_counts_and_indices():
     # packed order: text, condition video, condition audio, audio, video
     assert lay.token_tags.tolist() == [1] * 5 + [0] * 12 + [2] * 4 + [2] * 14 + [0] * 18
     assert lay.text_indices.tolist() == list(range(5))
-    assert lay.audio_indices.tolist() == list(range(21, 35))
-    assert lay.video_indices.tolist() == list(range(35, 53))
+    # the index sets cover a modality's condition rows first, then its targets (the wrapper concatenates them
+    # that way and checks the totals, src/pika_h3/core/wrapper.py:171-179)
+    assert lay.audio_indices.tolist() == list(range(17, 35))
+    assert lay.video_indices.tolist() == list(range(5, 17)) + list(range(35, 53))
+    assert lay.video_indices.numel() == c.condition_video + c.video and lay.audio_indices.numel() == c.condition_audio + c.audio
+    every = torch.cat([lay.text_indices, lay.video_indices, lay.audio_indices]).sort().values
+    assert every.tolist() == list(range(53))                      # a partition of the rows
     assert lay.num_condition_video_rows == 12 and lay.num_condition_audio_rows == 4 and lay.num_text_tokens == 5
     pos = lay.position_ids
     assert float(pos[:5].abs().sum()) == 0.0                       # text at position 0
@@ -102,3 +107,22 @@ def test_layout_cache_is_lru_by_geometry():
     cache.get(**{**g, "num_text_tokens": 5})        # evicts b
     assert cache.get(**{**g, "num_text_tokens": 4}) is not b
     assert cache.get(**{**g, "keyframe_frames": [1]}).counts.condition_video == 4
+
+
+def test_row_timesteps_per_segment():
+    """Unique timesteps + per-row index, with the argument list of src/pika_h3/core/packing.py:212-231 and the
+    values the wrapper passes (src/pika_h3/core/wrapper.py:182-190)."""
+    lay = P.build_layout(num_text_tokens=5, num_latent_frames=3, latent_height=4, latent_width=6,
+                         num_audio_latents=7, keyframe_frames=(0, 2), reference_audio_rows=4)
+    uniq, idx = P.row_timesteps(lay, video_t=0.25, audio_t=0.5, condition_video_t=max(0.25, 0.75), condition_audio_t=1.0)
+    assert uniq.dtype == torch.float32 and idx.dtype == torch.int32 and idx.shape == (53,)
+    assert uniq.tolist() == [0.25, 0.5, 0.75, 1.0]
+    per_row = uniq[idx.long()].tolist()
+    # text (clean), keyframe rows (pinned), condition audio (clean), audio, video
+    assert per_row == [1.0] * 5 + [0.75] * 12 + [1.0] * 4 + [0.5] * 14 + [0.25] * 18
+    # equal times share one entry: video and audio at the same time, keyframes no noisier than the video
+    uniq, idx = P.row_timesteps(lay, video_t=0.5, audio_t=0.5, condition_video_t=0.5)
+    assert uniq.tolist() == [0.5, 1.0] and idx.tolist() == [1] * 5 + [0] * 12 + [1] * 4 + [0] * 32
+    # the text switch
+    uniq, idx = P.row_timesteps(lay, video_t=0.5, audio_t=0.5, condition_video_t=0.5, condition_audio_t=0.5, text_t=0.5)
+    assert uniq.tolist() == [0.5] and int(idx.abs().sum()) == 0
