@@ -11,11 +11,12 @@ from .layout import (
     video_position_ids,
 )
 from . import packing
+from . import projections
 from .ops import BlockMask, attention, rope_tables, time_attention_kernel
 from .processor import PikaH3AttnProcessor
 
 __all__ = [
     "BlockMask", "PikaH3AttnProcessor", "Pkh3Error", "ROPE_HALF", "ROPE_INTERLEAVED", "ROPE_NONE",
-    "attention", "audio_position_ids", "local_window_tile_map", "packing", "rope_tables", "time_attention_kernel",
+    "attention", "audio_position_ids", "local_window_tile_map", "packing", "projections", "rope_tables", "time_attention_kernel",
     "video_position_ids",
 ]

@@ -20,6 +20,7 @@ import torch
 
 from . import _lib
 from .ops import BlockMask, attention, rope_tables
+from .projections import PackedLinear, adaln_modulate, out_proj, pack_rows, qkv_attention
 
 
 def _norm_weight(mod, dim: int, device) -> Optional[torch.Tensor]:
@@ -49,12 +50,19 @@ class PikaH3AttnProcessor:
         rope_theta: float = 10000.0,
         norm_eps: float = 1e-6,
         fp8_qk: bool = False,
+        fused_projections: bool = False,
+        lora_adapter: str = "default",
     ):
         self.rope_mode = int(rope_mode)
         self.rope_axes_dims = tuple(int(x) for x in rope_axes_dims)
         self.rope_theta = float(rope_theta)
         self.norm_eps = float(norm_eps)
         self.fp8_qk = bool(fp8_qk)
+        # self-attention of one document through the library's own projection GEMMs (LoRA as a second K segment,
+        # K/V written by the GEMM epilogue in the attention kernel's layout) instead of the module's torch GEMMs
+        self.fused_projections = bool(fused_projections)
+        self.lora_adapter = str(lora_adapter)
+        self._packed: Dict[int, Tuple[object, Dict[str, PackedLinear]]] = {}
         # position grids are constant across layers and denoising steps: one table per grid
         self._rope_cache: Dict[Hashable, Tuple[Optional[torch.Tensor], Tuple[torch.Tensor, torch.Tensor]]] = {}
         # one scratch buffer per (device, stream), grown on demand and reused by every layer call on that stream
@@ -88,6 +96,28 @@ class PikaH3AttnProcessor:
             self._workspaces[key] = ws
         return ws
 
+    def packed_weights(self, attn) -> Dict[str, PackedLinear]:
+        """The module's four projections as operand images, packed on first use and kept with the module (weights
+        are static at inference; call :meth:`forget` after changing them)."""
+        hit = self._packed.get(id(attn))
+        if hit is None or hit[0] is not attn:
+            packed = {
+                "q": PackedLinear.from_module(attn.to_q, adapter=self.lora_adapter),
+                "k": PackedLinear.from_module(attn.to_k, adapter=self.lora_adapter),
+                "v": PackedLinear.from_module(attn.to_v, head_perm=False, adapter=self.lora_adapter),
+                "out": PackedLinear.from_module(attn.to_out[0], adapter=self.lora_adapter),
+            }
+            hit = (attn, packed)
+            self._packed[id(attn)] = hit
+        return hit[1]
+
+    def forget(self, attn=None) -> None:
+        """Drop packed weights (of one module, or all)."""
+        if attn is None:
+            self._packed.clear()
+        else:
+            self._packed.pop(id(attn), None)
+
     def __call__(
         self,
         attn,
@@ -100,6 +130,10 @@ class PikaH3AttnProcessor:
         block_mask: Optional[BlockMask] = None,
         fp8_qk: Optional[bool] = None,
         rope_key: Optional[Hashable] = None,
+        adaln: Optional[dict] = None,
+        gate: Optional[torch.Tensor] = None,
+        gate_index: Optional[torch.Tensor] = None,
+        residual: Optional[torch.Tensor] = None,
     ) -> torch.Tensor:
         """``hidden_states [B, S, H*D]`` -> ``[B, S, H*D]``.
 
@@ -109,11 +143,24 @@ class PikaH3AttnProcessor:
         [S, 3]`` (or precomputed ``rope_cos_sin`` fp32 ``[S, D/2]`` tables); ``rope_key`` names the grid for the
         table cache (see :meth:`_tables`).  The softmax scale is ``attn.scale`` when the module has one, else
         ``1/sqrt(D)``.  fp8 QK^T is not defined together with a key mask: such a call runs in bf16.
+
+        With ``fused_projections`` (self-attention, B = 1, no mask) the projections run in the library too, and the
+        block's surroundings can ride along: ``adaln = dict(shift=, scale=, row_index=, norm=, eps=)`` applies
+        ``norm(x) * (1 + scale[row_index]) + shift[row_index]`` to ``hidden_states`` before ``to_q/to_k/to_v``
+        (patches/0001-h3-adaln-fp32.patch:34-40), and ``gate`` (bf16 ``[rows, C]``, gathered by ``gate_index``,
+        int32 ``[S]``) and ``residual`` (``[B, S, C]``) make the result ``residual + gate * to_out(...)``.
+        Without ``fused_projections`` those three arguments are rejected.
         """
         if hidden_states.dim() != 3:
             raise ValueError(f"hidden_states must be [B, S, C], got {tuple(hidden_states.shape)}")
         B, S, _ = hidden_states.shape
         H = int(attn.heads)
+        fused = self.fused_projections and encoder_hidden_states is None and attention_mask is None and B == 1
+        if not fused and (adaln is not None or gate is not None or residual is not None):
+            raise ValueError("adaln / gate / residual need fused_projections, self-attention, B = 1 and no mask")
+        if fused:
+            return self._fused(attn, hidden_states, position_ids=position_ids, rope_cos_sin=rope_cos_sin, block_mask=block_mask,
+                               fp8_qk=fp8_qk, rope_key=rope_key, adaln=adaln, gate=gate, gate_index=gate_index, residual=residual)
         kv_src = hidden_states if encoder_hidden_states is None else encoder_hidden_states
         q = attn.to_q(hidden_states)
         k = attn.to_k(kv_src)
@@ -156,3 +203,36 @@ class PikaH3AttnProcessor:
         if len(attn.to_out) > 1:
             out = attn.to_out[1](out)
         return out
+
+    def _fused(self, attn, hidden_states, *, position_ids, rope_cos_sin, block_mask, fp8_qk, rope_key, adaln, gate, gate_index,
+               residual) -> torch.Tensor:
+        _, S, C = hidden_states.shape
+        H = int(attn.heads)
+        if C != H * 128:
+            raise ValueError(f"hidden size {C} is not heads x 128")
+        x = hidden_states[0]
+        if x.dtype != torch.bfloat16:
+            x = x.to(torch.bfloat16)
+        packed = self.packed_weights(attn)
+        x_img = pack_rows(x) if adaln is None else adaln_modulate(x, **adaln)
+        qn, kn = getattr(attn, "norm_q", None), getattr(attn, "norm_k", None)
+        eps = getattr(qn, "eps", None)
+        scale = getattr(attn, "scale", None)
+        opts = dict(
+            q_norm_weight=_norm_weight(qn, 128, x.device), k_norm_weight=_norm_weight(kn, 128, x.device),
+            norm_eps=self.norm_eps if eps is None else float(eps),
+            fp8_qk=self.fp8_qk if fp8_qk is None else bool(fp8_qk), block_mask=block_mask,
+            softmax_scale=None if scale is None else float(scale),
+        )
+        if rope_cos_sin is None and position_ids is not None:
+            rope_cos_sin = self._tables(position_ids, rope_key)
+        if rope_cos_sin is not None:
+            opts.update(rope_mode=self.rope_mode, rope_q=rope_cos_sin, rope_k=rope_cos_sin)
+        o = qkv_attention(x_img, S, packed["q"], packed["k"], packed["v"], heads=H, **opts)
+        res = None
+        if residual is not None:
+            res = residual[0] if residual.dim() == 3 else residual
+            if res.dtype != torch.bfloat16:
+                res = res.to(torch.bfloat16)
+        y = out_proj(o.view(S, C), packed["out"], gate=gate, row_index=gate_index, residual=res)
+        return y.view(1, S, C).to(hidden_states.dtype)

@@ -213,3 +213,114 @@ def PackedLinear_from(d, head_perm=True):
 
     return PackedLinear.from_weights(d["weight"], d.get("bias"), lora_a=d.get("lora_a"), lora_b=d.get("lora_b"),
                                      lora_scale=d.get("lora_scale", 1.0), head_perm=head_perm)
+
+
+class _LoraLinear(torch.nn.Module):
+    """What PEFT's ``add_adapter`` leaves on a target (src/pika_h3/core/loader.py:36-37): the base layer plus
+    ``lora_A`` / ``lora_B`` / ``scaling`` per adapter name, applied as base(x) + scaling * B(A(x))."""
+
+    def __init__(self, n_in, n_out, rank=128, alpha=64, bias=True):
+        super().__init__()
+        self.base_layer = torch.nn.Linear(n_in, n_out, bias=bias)
+        self.lora_A = torch.nn.ModuleDict({"default": torch.nn.Linear(n_in, rank, bias=False)})
+        self.lora_B = torch.nn.ModuleDict({"default": torch.nn.Linear(rank, n_out, bias=False)})
+        self.scaling = {"default": alpha / rank}
+        torch.nn.init.normal_(self.lora_B["default"].weight, std=0.05)
+
+    def forward(self, x):
+        return self.base_layer(x) + self.scaling["default"] * self.lora_B["default"](self.lora_A["default"](x))
+
+
+class _Attn(torch.nn.Module):
+    def __init__(self, hidden, heads, lora):
+        super().__init__()
+        self.heads = heads
+        mk = (lambda: _LoraLinear(hidden, hidden)) if lora else (lambda: torch.nn.Linear(hidden, hidden))
+        self.to_q, self.to_k, self.to_v = mk(), mk(), mk()
+        self.to_out = torch.nn.ModuleList([mk(), torch.nn.Identity()])
+        self.norm_q = torch.nn.RMSNorm(hidden // heads, eps=1e-6)
+        self.norm_k = torch.nn.RMSNorm(hidden // heads, eps=1e-6)
+
+
+@pytest.mark.parametrize("lora", [False, True])
+def test_processor_with_fused_projections(lora):
+    """The processor with the library's projections (packed from the module, LoRA wrapper included) against the same
+    processor on the module's own torch GEMMs, and the block extras (AdaLN, gate, residual) against the oracle."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as AO
+    from oracle import projection_oracle as PO
+
+    torch.manual_seed(5)
+    H, hidden, S = 3, 384, 410
+    attn = _Attn(hidden, H, lora).cuda().to(torch.bfloat16)
+    x = torch.randn((1, S, hidden), device="cuda", dtype=torch.bfloat16)
+    pos = torch.cat([pk.video_position_ids(2, 10, 20), pk.audio_position_ids(5)], 0).cuda()
+    plain, fused = pk.PikaH3AttnProcessor(), pk.PikaH3AttnProcessor(fused_projections=True)
+    with torch.no_grad():
+        y0 = plain(attn, x, position_ids=pos)
+        y1 = fused(attn, x, position_ids=pos)
+    torch.cuda.synchronize()
+    err, cos = AO.max_abs_and_cosine(y1.cpu(), y0.cpu())
+    print(f"fused vs torch projections (lora={lora}): max_abs={err:.3e} cos={cos:.8f}", flush=True)
+    assert y1.shape == x.shape and err <= 3e-2 and cos >= 0.9999
+    assert fused.packed_weights(attn) is fused.packed_weights(attn)          # packed once
+    # block extras against the oracle
+    T = 2
+    shift, scale, gate = (torch.randn((T, hidden), device="cuda").mul(0.2).to(torch.bfloat16) for _ in range(3))
+    idx = (torch.arange(S, device="cuda") % T).to(torch.int32)
+    with torch.no_grad():
+        y2 = fused(attn, x, position_ids=pos, adaln=dict(shift=shift, scale=scale, row_index=idx, norm="layer"),
+                   gate=gate, gate_index=idx, residual=x)
+    torch.cuda.synchronize()
+
+    def lin_of(mod):
+        base = getattr(mod, "base_layer", mod)
+        d = dict(weight=base.weight.detach().cpu(), bias=base.bias.detach().float().cpu())
+        if lora:
+            d.update(lora_a=mod.lora_A["default"].weight.detach().cpu(), lora_b=mod.lora_B["default"].weight.detach().cpu(),
+                     lora_scale=mod.scaling["default"])
+        return d
+
+    lin = {"q": lin_of(attn.to_q), "k": lin_of(attn.to_k), "v": lin_of(attn.to_v), "out": lin_of(attn.to_out[0])}
+    ref = PO.attention_block(x[0].cpu(), lin, heads=H, shift=shift.cpu(), scale=scale.cpu(), gate=gate.cpu(), row_index=idx.cpu(),
+                             q_norm_weight=attn.norm_q.weight.float().cpu(), k_norm_weight=attn.norm_k.weight.float().cpu(),
+                             rope_mode=AO.ROPE_INTERLEAVED, rope_q=AO.rope_tables(pos.cpu()))
+    err, cos = AO.max_abs_and_cosine(y2[0].cpu(), ref["y"])
+    print(f"fused block with AdaLN, gate, residual (lora={lora}): max_abs={err:.3e} cos={cos:.8f}", flush=True)
+    assert err <= 2e-2 * max(1.0, float(ref["y"].abs().max())) and cos >= 0.9999
+    with pytest.raises(ValueError):
+        plain(attn, x, position_ids=pos, gate=gate)
+
+
+def test_rope_cache_tells_two_grids_of_equal_length_apart():
+    """Two geometries with the same token count (landscape and portrait), allocated one after the other as the
+    reference builds a fresh layout per forward: each call must see its own tables."""
+    import pika_h3_flex_amd as pk
+
+    torch.manual_seed(6)
+    H, hidden = 2, 256
+    attn = _Attn(hidden, H, False).cuda().to(torch.bfloat16)
+    S = 6 * 10
+    x = torch.randn((1, S, hidden), device="cuda", dtype=torch.bfloat16)
+    proc, fresh = pk.PikaH3AttnProcessor(), pk.PikaH3AttnProcessor()
+    outs = []
+    for hp, wp in ((6, 10), (10, 6)):
+        pos = pk.video_position_ids(1, hp, wp).cuda()          # same S, same allocator slot once the first is freed
+        with torch.no_grad():
+            outs.append((proc(attn, x, position_ids=pos), pk.PikaH3AttnProcessor()(attn, x, position_ids=pos)))
+        del pos
+    torch.cuda.synchronize()
+    for got, want in outs:
+        assert torch.equal(got, want)
+    assert not torch.equal(outs[0][0], outs[1][0])
+    # an in-place edit of a cached grid is seen as a new grid; a caller-supplied key short-cuts the identity check
+    pos = pk.video_position_ids(1, 6, 10).cuda()
+    with torch.no_grad():
+        a = proc(attn, x, position_ids=pos)
+        pos[:, 2] += 3.0
+        pos[:, 1] *= 2.0
+        b = proc(attn, x, position_ids=pos)
+        c = fresh(attn, x, position_ids=pos)
+        d = proc(attn, x, position_ids=pos, rope_key=("landscape", 6, 10, "edited"))
+    torch.cuda.synchronize()
+    assert torch.equal(b, c) and torch.equal(d, c) and not torch.equal(a, b)
