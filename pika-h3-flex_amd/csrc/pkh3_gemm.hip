@@ -8,7 +8,7 @@
 // Operands.  Both operands come as 1 KiB operand images (32 rows x 16 contraction elements, lane l holds row
 // l%32, elements 8*(l/32)..+7): activations as [token block][k-step], weights as [feature block][k-step] (packed
 // once when the weights are loaded).  They move HBM/L2 -> LDS -> VGPR as straight 16-byte copies, like the K/V
-// tiles of the attention kernel: direct-to-LDS loads into a 3-slot ring, two chunks ahead, one barrier per chunk.
+// tiles of the attention kernel: direct-to-LDS loads into a 4-slot ring, three chunks ahead, one barrier per chunk.
 // Since the two MFMA operands have the same register form, one pair of images serves both orientations:
 //   C^T = W x^T  (features down the accumulator registers, one token per lane)   Q, K, row-major outputs
 //   C   = x W^T  (tokens down the registers, one feature per lane)               V images
@@ -29,7 +29,7 @@ constexpr int kGemmWaves = 8;
 constexpr int kGemmTile = 256;                      // tokens and features per workgroup
 constexpr int kGemmChunkK = 32;                     // contraction elements per ring slot
 constexpr int kGemmStageBytes = 2 * kGemmTile * kGemmChunkK * 2;  // weight part + activation part
-constexpr int kGemmRing = 3;
+constexpr int kGemmRing = 4;
 
 __device__ __forceinline__ void gemm_dma16(const char* g, unsigned lane_off, char* l) {
   // see lds_dma16 in pkh3_attn_fwd.hip: wave-uniform base addresses, per-lane byte offset, tracked by vmcnt
@@ -87,33 +87,53 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[t2][db][i] = 0.f;
 
-  dma(0, 0);
-  if (nk > 1) dma(1, 1);
-  int slot = 0, slot_prev = kGemmRing - 1;
+  // Ring of four chunks.  Entering iteration kc: chunk kc is in LDS for every wave and its first k-step's images are
+  // already on their way to this wave's registers; chunks kc+1 and kc+2 are in flight.  The barrier at the top makes
+  // chunk kc+1 visible and frees the slot of chunk kc-1 for chunk kc+3, so the first images of the next chunk can be
+  // read at the tail of this iteration and no wave starts a chunk by waiting for LDS.
+  const int n_pre = nk < 3 ? nk : 3;
+  for (int c = 0; c < n_pre; ++c) dma(c, c);
+  if (n_pre == 3) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if (n_pre == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  const int w_off = (fh * 4) * 2048 + lane * 16;            // weight blocks fh*4..+3 of a slot
+  const int a_off = 16384 + (tq * 2) * 2048 + lane * 16;    // token blocks tq*2, +1
+  bf16x8 wf[2][4], xf[2][2];
+  auto read_frags = [&](int slot, int ks, bf16x8 (&w4)[4], bf16x8 (&x2)[2]) {
+    const char* base = lds_raw + slot * kGemmStageBytes + ks * 1024;
+#pragma unroll
+    for (int db = 0; db < 4; ++db) w4[db] = *(const bf16x8*)(base + w_off + db * 2048);
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) x2[t2] = *(const bf16x8*)(base + a_off + t2 * 2048);
+  };
+  auto mfma8 = [&](const bf16x8 (&w4)[4], const bf16x8 (&x2)[2]) {
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        if constexpr (EPI == kEpiVImg) acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x2[t2], w4[db], acc[t2][db], 0, 0, 0);
+        else acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w4[db], x2[t2], acc[t2][db], 0, 0, 0);
+      }
+  };
+  if (head_live) read_frags(0, 0, wf[0], xf[0]);
+  int slot = 0;
   for (int kc = 0; kc < nk; ++kc) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    const char* wbuf = lds_raw + slot * kGemmStageBytes + (fh * 4) * 2048;           // weight blocks fh*4..+3
-    const char* abuf = lds_raw + slot * kGemmStageBytes + 16384 + (tq * 2) * 2048;   // token blocks tq*2, +1
-    if (kc + 2 < nk) dma(kc + 2, slot_prev);
-    slot_prev = slot;
-    slot = slot == kGemmRing - 1 ? 0 : slot + 1;
-    if (!head_live) continue;  // wave-uniform: a head past the end of the target (barriers and copies still run)
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      bf16x8 wf[4], xf[2];
-#pragma unroll
-      for (int db = 0; db < 4; ++db) wf[db] = *(const bf16x8*)(wbuf + (db * 2 + ks) * 1024 + lane * 16);
-#pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) xf[t2] = *(const bf16x8*)(abuf + (t2 * 2 + ks) * 1024 + lane * 16);
-#pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          if constexpr (EPI == kEpiVImg) acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[t2], wf[db], acc[t2][db], 0, 0, 0);
-          else acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[db], xf[t2], acc[t2][db], 0, 0, 0);
-        }
+    if (kc + 1 < nk) {
+      // chunk kc+1 has landed (this wave's pieces; the barrier covers the others'); only chunk kc+2's copies may be pending
+      if (kc + 2 < nk) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (kc + 3 < nk) dma(kc + 3, (slot + 3) & 3);
     }
+    const int next = (slot + 1) & 3;
+    if (head_live) {  // wave-uniform: a head past the end of the target only copies and synchronises
+      read_frags(slot, 1, wf[1], xf[1]);
+      mfma8(wf[0], xf[0]);
+      if (kc + 1 < nk) read_frags(next, 0, wf[0], xf[0]);
+      mfma8(wf[1], xf[1]);
+    }
+    slot = next;
   }
   // let the last MFMA retire before anything the compiler places after the loop reads the accumulators
   asm volatile("s_nop 15\n\ts_nop 15"
@@ -246,14 +266,25 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
 
 __global__ __launch_bounds__(64 * kGemmWaves, 1) void gemm_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(1024))) char lds_raw[kGemmRing * kGemmStageBytes];
-  // Workgroups go to the 8 XCDs round-robin; each XCD takes one contiguous run of (token tile, feature tile)
-  // with the feature tile varying fastest, so the CUs behind one L2 share a token tile's activations.
+  // Workgroups go to the 8 XCDs round-robin; each XCD takes one contiguous run of the tile order below, in which 32
+  // consecutive tiles (the workgroups the 32 CUs behind one L2 run together) form a block of 4 token tiles x 8
+  // feature tiles: every activation panel is then shared by 8 and every weight panel by 4 of them.
+  constexpr int kBlockN = 8;
   const int total = p.m_tiles * p.n_tiles;
   const int per_xcd = (total + 7) / 8;
   const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (lin >= total) return;
-  const int m_tile = lin / p.n_tiles;
-  int n_tile = lin % p.n_tiles;
+  const int full = p.n_tiles / kBlockN * kBlockN;       // feature tiles in whole column blocks
+  int m_tile, n_tile;
+  if (lin < full * p.m_tiles) {
+    const int nb = lin / (kBlockN * p.m_tiles), rem = lin % (kBlockN * p.m_tiles);
+    m_tile = rem / kBlockN;
+    n_tile = nb * kBlockN + rem % kBlockN;
+  } else {
+    const int rest = lin - full * p.m_tiles, width = p.n_tiles - full;
+    m_tile = rest / width;
+    n_tile = full + rest % width;
+  }
   int t = 0;
   while (t + 1 < p.n_targets && n_tile >= p.tg[t].n_tiles) { n_tile -= p.tg[t].n_tiles; ++t; }
   const GemmTarget& tg = p.tg[t];
