@@ -51,12 +51,129 @@ def host_cpu():
     return model, (len(cores) or os.cpu_count() or 0)
 
 
+def _time_steps(step, steps, warmup):
+    """(mean ms per step over the K timed steps bracketed by synchronisation, median, minimum)."""
+    import torch
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    marks[0].record()
+    for i in range(steps):
+        step()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    mean = (time.perf_counter() - t0) * 1e3 / steps
+    per = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    return mean, per[len(per) // 2], per[0]
+
+
+def bench_block(args, pk, workloads, dev) -> int:
+    """The attention half of one DiT block at 480p: AdaLN modulation -> to_q/to_k/to_v (+LoRA rank 128) -> attention ->
+    to_out.0 (+LoRA) with gate and residual.  A "step" is that whole sequence through the library's projection GEMMs
+    (K/V written by the GEMM epilogue in the attention kernel's layout); the same block with the projections and the
+    modulation as torch ops (hipBLASLt GEMMs, then the library's K/V pass and attention kernel) is timed beside it."""
+    import torch
+    import torch.nn.functional as F
+
+    from pika_h3_flex_amd import projections as P
+
+    blk = workloads.block_inputs(frames=31, rows_h=30, rows_w=52, seed=args.seed, device=dev, name="480p-block")
+    S, C = blk.x.shape
+    H = blk.heads
+    ones = torch.ones(128, dtype=torch.float32, device=dev)
+    tabs = pk.rope_tables(blk.position_ids)
+    opts = dict(q_norm_weight=ones, k_norm_weight=ones, norm_eps=1e-6, rope_mode=pk.ROPE_INTERLEAVED, rope_q=tabs)
+    packed = {n: P.PackedLinear.from_weights(d["weight"], d["bias"], lora_a=d["lora_a"], lora_b=d["lora_b"],
+                                             lora_scale=d["lora_scale"], head_perm=(n != "v")) for n, d in blk.linears.items()}
+
+    def fused():
+        x_img = P.adaln_modulate(blk.x, shift=blk.shift, scale=blk.scale, row_index=blk.row_index, norm="layer")
+        o = P.qkv_attention(x_img, S, packed["q"], packed["k"], packed["v"], heads=H, **opts)
+        return P.out_proj(o.view(S, C), packed["out"], gate=blk.gate, row_index=blk.row_index, residual=blk.x)
+
+    idx = blk.row_index.long()
+
+    def lin(x, d):
+        return F.linear(x, d["weight"], d["bias"].to(x.dtype)) + d["lora_scale"] * F.linear(F.linear(x, d["lora_a"]), d["lora_b"])
+
+    def unfused():
+        xm = F.layer_norm(blk.x, (C,), eps=1e-6) * (1 + blk.scale.index_select(0, idx)) + blk.shift.index_select(0, idx)
+        q, k, v = (lin(xm, blk.linears[n]).view(1, S, H, 128) for n in ("q", "k", "v"))
+        o = pk.attention(q, k, v, **opts)
+        return blk.x + blk.gate.index_select(0, idx) * lin(o.view(S, C), blk.linears["out"])
+
+    def projections_only():
+        x_img = P.adaln_modulate(blk.x, shift=blk.shift, scale=blk.scale, row_index=blk.row_index, norm="layer")
+        return x_img
+
+    ms, ms_median, ms_min = _time_steps(fused, args.steps, args.warmup)
+    ms_unfused, _, _ = _time_steps(unfused, max(3, args.steps // 4), 2)
+    # the GEMM launches alone: QKV (+ down-projections) and to_out, events on the launch stream
+    x_img = P.adaln_modulate(blk.x, shift=blk.shift, scale=blk.scale, row_index=blk.row_index, norm="layer")
+    o = torch.randn((S, C), device=dev).to(torch.bfloat16)
+    q_scratch = torch.empty((1, S, H, 128), dtype=torch.bfloat16, device=dev)
+
+    def qkv_only():
+        import ctypes as C_
+
+        from pika_h3_flex_amd import _lib
+
+        a, keep = pk.ops.fill_args(q_scratch, None, None, torch.empty_like(q_scratch), kv_prepared=True, **opts)
+        ws = torch.empty(pk.ops.workspace_bytes(a), dtype=torch.uint8, device=dev)
+        lws = torch.empty(P.packed_bytes(S, 3 * _lib.LORA_RANK), dtype=torch.uint8, device=dev)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+        pa = _lib.QkvArgs()
+        pa.x_img, pa.S, pa.K = x_img.data_ptr(), S, C
+        pa.q, pa.k, pa.v = packed["q"].c_struct(), packed["k"].c_struct(), packed["v"].c_struct()
+        pa.lora_workspace, pa.lora_workspace_bytes = lws.data_ptr(), lws.numel()
+        st = C_.c_void_p(torch.cuda.current_stream().cuda_stream)
+        lib = _lib.load()
+
+        def run():
+            _lib.check(lib.pkh3_qkv_proj(C_.byref(pa), C_.byref(a), st))
+        return run, (ws, lws, keep)
+
+    run_qkv, _keep = qkv_only()
+    ms_qkv, _, _ = _time_steps(run_qkv, 10, 3)
+    ms_out, _, _ = _time_steps(lambda: P.out_proj(o, packed["out"], gate=blk.gate, row_index=blk.row_index, residual=blk.x), 10, 3)
+    ms_mod, _, _ = _time_steps(projections_only, 10, 3)
+    r = blk.linears["q"]["lora_a"].shape[0]
+    flops_qkv = 3 * (2.0 * S * C * C + 2.0 * S * C * r + 2.0 * S * r * C)
+    flops_out = 2.0 * S * C * C + 2.0 * S * C * r + 2.0 * S * r * C
+    total = blk.attention_flops + blk.projection_flops
+    value = total / (ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS["bf16"]
+    gemm_tflops = flops_qkv / (ms_qkv * 1e-3) / 1e12
+    line = {
+        "metric": "attention-block TFLOP/s (attention 4*S*S*D*H + the four projections with LoRA; AdaLN, gate and residual included in the time)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"480p attention block: S={S}, hidden={C}, H={H}, D=128, LoRA rank {r} on to_q/to_k/to_v/to_out.0, "
+                               f"AdaLN over {blk.shift.shape[0]} timestep groups, QK-RMSNorm + 3-axis RoPE, non-causal",
+                   "seed": args.seed, "ms_per_step_median": round(ms_median, 4), "ms_per_step_min": round(ms_min, 4),
+                   "ms_per_step_with_torch_projections": round(ms_unfused, 4),
+                   "ms_adaln_modulate": round(ms_mod, 4), "ms_qkv_projection": round(ms_qkv, 4),
+                   "ms_out_projection_with_packing": round(ms_out, 4),
+                   "out_projection_tflops": round(flops_out / (ms_out * 1e-3) / 1e12, 2)},
+        "roofline": {"bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(gemm_tflops / peak, 4), "traffic": None, "kernel": "gemm_kernel (to_q/to_k/to_v + LoRA, two launches)",
+                     "kernel_ms": round(ms_qkv, 4), "flops_per_launch": flops_qkv},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="480p", choices=["plumbing", "480p", "768p", "joint", "cross", "480p-sparse", "480p-sparse-fp8", "480p-fp8"])
+    ap.add_argument("--workload", default="480p", choices=["plumbing", "480p", "768p", "joint", "cross", "480p-sparse", "480p-sparse-fp8", "480p-fp8", "480p-block"])
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-rows", type=int, default=32768, help="query rows of the CPU baseline sample (0 = skip)")
     ap.add_argument("--kernel-iters", type=int, default=10)
@@ -81,6 +198,9 @@ def main() -> int:
         return 2
     dev = "cuda:0"
     torch.cuda.set_device(0)
+
+    if args.workload == "480p-block":
+        return bench_block(args, pk, workloads, dev)
 
     base = args.workload.split("-")[0]
     inp = workloads.make(base, seed=args.seed, device=dev)
@@ -137,10 +257,18 @@ def main() -> int:
     kernel_ms = pk.time_attention_kernel(inp.q, inp.k, inp.v, iters=args.kernel_iters, **opts)
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS["fp8" if fp8 else "bf16"]
+    traffic = MEASURED_TRAFFIC.get(args.workload, (None, None))[0]
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
                 "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1], "kernel": "attn_fwd_kernel",
                 "kernel_ms": round(kernel_ms, 4), "flops_per_launch": flops}
+
+    if traffic is not None:
+        # the other roof: bytes that crossed the L2 boundary per launch (profiled) over this run's kernel time
+        rate = traffic / (kernel_ms * 1e-3) / 1e9
+        roofline["traffic_rate_gbs"] = round(rate, 1)
+        roofline["traffic_frac_of_hbm_peak"] = round(rate / HBM_PEAK_GBS, 4)
+        roofline["binding_roof"] = "hbm" if rate / HBM_PEAK_GBS > achieved / peak else "mfma"
 
     cpu = None
     if args.cpu_rows > 0:

@@ -96,8 +96,8 @@ WsPlan plan(const pkh3_attn_args* a) {
   w.kscale_off = off; if (fp8) off = align_up(off + bh * w.nKt * sizeof(float), 256);
   w.cnt_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * sizeof(int), 256);
   w.idx_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * a->Sk * sizeof(int), 256);
-  w.plan_off = off;   if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / 4) * 5 * w.nKt * sizeof(int), 256);
-  w.plan_cnt_off = off; if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / 4) * 5 * sizeof(int), 256);
+  w.plan_off = off;   if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / kSparseRows) * kSparseLists * w.nKt * sizeof(int), 256);
+  w.plan_cnt_off = off; if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / kSparseRows) * kSparseLists * sizeof(int), 256);
   w.kmax_off = off;   off = align_up(off + bh * sizeof(float), 256);
   w.total = off;
   return w;
@@ -154,7 +154,7 @@ void build(const pkh3_attn_args* a, void* workspace, Launch& L) {
   f.c = scale * kLog2e;
   f.plan = a->blk_row_ptr ? (const int*)(ws + L.w.plan_off) : nullptr;
   f.plan_cnt = a->blk_row_ptr ? (const int*)(ws + L.w.plan_cnt_off) : nullptr;
-  f.plan_stride = 5 * L.w.nKt;
+  f.plan_stride = kSparseLists * L.w.nKt;
   f.kscale = k.scale_out; f.fp8 = fp8; f.long_key_kernel = (a->flags & PKH3_FLAG_LONG_KEY_KERNEL) ? 1 : 0;
   f.kmax = (const float*)(ws + L.w.kmax_off);
 }
@@ -171,7 +171,7 @@ int run_prologue(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
   if (a->blk_row_ptr) {
     char* ws = L.ws;
     if ((e = launch_sparse_plan(a->blk_row_ptr, a->blk_col_idx, (a->Sq + 63) / 64, L.w.nQ64, L.w.nKt, (int*)(ws + L.w.plan_off),
-                                5 * L.w.nKt, (int*)(ws + L.w.plan_cnt_off), st)) != hipSuccess)
+                                kSparseLists * L.w.nKt, (int*)(ws + L.w.plan_cnt_off), st)) != hipSuccess)
       return hip_fail(e, "sparse plan");
   }
   if (a->flags & PKH3_FLAG_KV_PREPARED) return PKH3_OK;  // pkh3_qkv_proj wrote K, V, the scales and the row-norm maxima

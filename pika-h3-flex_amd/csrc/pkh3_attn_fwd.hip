@@ -42,7 +42,7 @@ namespace pkh3 {
 constexpr int kDenseWaves = 12;  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
 constexpr int kShortWaves = 4;   // short-key dense kernel: three 4-wave workgroups per CU
 constexpr int kShortMaxTiles = 16;  // key tiles up to which the short-key kernel is used
-constexpr int kSparseWaves = 8;  // the block-sparse kernel is built around 4 row-blocks x 2 waves (two per SIMD)
+constexpr int kSparseWaves = 2 * kSparseRows;  // block-sparse: a wave pair per row-block; two such workgroups share a CU
 constexpr int kRing = 3;               // LDS ring depth (tiles)
 constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
 constexpr float kStaticMaxLimit = 48.0f;  // rows whose |logit| bound is below this skip the running max (terms 2^-48 .. 2^48)
@@ -361,9 +361,14 @@ __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int 
 // per group), then add their partial results up through LDS.  Such a workgroup lasts a third as long, so the
 // CUs that would idle through a whole round of whole workgroups idle through a third of one.
 template <bool FP8, bool SPARSE, int WAVES, bool SPLIT = false>
-__global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void attn_fwd_kernel(FwdParams p) {
-  static_assert(!SPARSE || WAVES == kSparseWaves, "block-sparse layout assumes 8 waves per workgroup");
-  constexpr bool SHORT = WAVES == kShortWaves;
+__global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWaves ? 3 : 1)) void attn_fwd_kernel(FwdParams p) {
+  static_assert(!SPARSE || WAVES == kSparseWaves, "block-sparse layout: a wave pair per row-block of the plan");
+  constexpr bool SHORT = !SPARSE && WAVES == kShortWaves;
+  constexpr bool LEAN = !SPARSE;                        // dense long-key form: three waves per SIMD, lean read-ahead
+  // whole-tile ring depth: three tiles, except where two workgroups share the CU's LDS and a bf16 tile is 32 KiB
+  constexpr int kRingT = (SPARSE && !FP8 && WAVES < 8) ? 2 : kRing;
+  constexpr int kAhead = kRingT - 1;                    // tiles in flight ahead of the one being used
+  constexpr int kStages2 = (SPARSE && FP8 && WAVES < 8) ? 3 : 2;  // sparse phase 2: stages of row-private half tiles
   constexpr bool HALFMODE = SHORT || SPLIT;             // rings of 32-key half tiles, 4 waves per ring
   constexpr int GROUPS = SPLIT ? WAVES / kShortWaves : 1;  // key-range groups of the workgroup
   static_assert(!(HALFMODE && SPARSE), "the half-tile forms are dense only");
@@ -372,10 +377,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
   constexpr int kTileBytes = kKBytes + kVTileBytes;
   constexpr int kChunks = kTileBytes / 1024;  // 1 KiB pieces of a tile, dealt round-robin to the waves
   constexpr int kHalfBytes = kTileBytes / 2;  // K and V images of 32 keys
-  // dense / phase 1: ring of kRing whole tiles; sparse phase 2: two stages of four row-private half tiles
+  // dense / phase 1: ring of kRingT whole tiles; sparse phase 2: kStages2 stages of row-private half tiles
   constexpr int kStageBytes = 32 * kD * 2;    // one wave's 32 x 128 bf16 output block, staged for the row-wise store
+  constexpr int kPhase2Bytes = SPARSE ? kStages2 * kSparseRows * kHalfBytes : 0;
   constexpr int kRingBytes = HALFMODE ? GROUPS * kRing * kHalfBytes
-                             : (SPARSE && 8 * kHalfBytes > kRing * kTileBytes ? 8 * kHalfBytes : kRing * kTileBytes);
+                             : (kPhase2Bytes > kRingT * kTileBytes ? kPhase2Bytes : kRingT * kTileBytes);
   constexpr int kMergeBytes = 64 * 64 * 4 + 2 * 64 * 4;  // SPLIT: one wave's O^T, row sums and row maxima in fp32
   constexpr int kAfterBytes = SPLIT ? kShortWaves * kMergeBytes : WAVES * kStageBytes;  // LDS use after the loops
   constexpr int kLdsBytes = kRingBytes > kAfterBytes ? kRingBytes : kAfterBytes;
@@ -411,9 +417,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
 
   const int sk = p.row_cnt ? p.row_cnt[b] : p.Sk;
   const int nkt = (sk + kTileKeys - 1) / kTileKeys;
-  // sparse: [tiles every row-block of this workgroup keeps | tiles only row-block 0 keeps | ... 1 | 2 | 3]
+  // sparse: [tiles every row-block of this workgroup keeps | tiles only row-block 0 keeps | ... 1 | ...]
   const int* plan = SPARSE ? p.plan + (int64_t)qt * p.plan_stride : nullptr;
-  const int* plan_cnt = SPARSE ? p.plan_cnt + qt * 5 : nullptr;
+  const int* plan_cnt = SPARSE ? p.plan_cnt + qt * kSparseLists : nullptr;
   const int nt = SPARSE ? uniform_load(plan_cnt, 0) : nkt;  // tiles all 8 waves walk together
 
   // this wave's pieces of every [K|V] tile record: 1 KiB chunks wave, wave + WAVES, ...
@@ -458,7 +464,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
     if (n_mine > 1) dma_short(h_begin + 1, 1);
   } else if (nt > 0) {
     dma(entry(0), 0);
-    if (nt > 1) dma(entry(1), 1);
+    if (kAhead > 1 && nt > 1) dma(entry(1), 1);
   }
   // Q load, fused with QK-RMSNorm, rotation and (fp8) quantisation: lane (l%32, hh) reads the 64 elements
   // d = 16*ks + 8*hh + j of query row q32*32 + l%32 -- the ones it carries in the MFMA B images -- so the
@@ -528,25 +534,25 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
     static_max = __all(bound <= kStaticMaxLimit);
   }
 
-  int slot = 0, slot_prev = kRing - 1;  // ring slots of tile i and of tile i-1 (the one tile i+2 is copied into)
+  int slot = 0, slot_prev = (HALFMODE ? kRing : kRingT) - 1;  // ring slots of tile i and of tile i-1 (which takes the newest copy)
   // Only the last key tile can be partial.  It is peeled off the loop so that the loop body has no masking
   // branch between S^T and the softmax, which lets the numerators of the first 32 keys be scheduled under
   // the MFMAs of the second 32.
   const int n_masked = (tail && nt > 0 && entry(nt - 1) == nkt - 1) ? 1 : 0;
 #define PKH3_TILE_LOOP(STATIC, MASKED, FROM, TO)                                                        \
   for (int i = FROM; i < TO; ++i) {                                                                     \
-    /* tiles i and i+1 are in LDS for every wave (own slices: vmcnt, the others': barrier), and every */ \
-    /* wave is past tile i-1, whose slot takes tile i+2 */                                              \
+    /* tile i (and, with a ring of three, i+1) is in LDS for every wave (own slices: vmcnt, the others': */ \
+    /* barrier), and every wave is past tile i-1, whose slot takes the newest copy */                   \
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
     __syncthreads();                                                                                    \
     const char* kbuf = lds[slot];                                                                       \
-    if (i + 2 < nt) dma(entry(i + 2), slot_prev);                                                       \
+    if (i + kAhead < nt) dma(entry(i + kAhead), slot_prev);                                             \
     slot_prev = slot;                                                                                   \
-    slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
+    slot = slot == kRingT - 1 ? 0 : slot + 1;                                                           \
     const int tile = entry(i);                                                                          \
-    qk_tile<FP8, (WAVES != kSparseWaves)>(w, kbuf, kbuf + kKBytes, lane);                                           \
+    qk_tile<FP8, LEAN>(w, kbuf, kbuf + kKBytes, lane);                                                  \
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
-    softmax_pv_tile<FP8, STATIC, (WAVES != kSparseWaves), MASKED>(w, kbuf + kKBytes, ct, tail, lane);                 \
+    softmax_pv_tile<FP8, STATIC, LEAN, MASKED>(w, kbuf + kKBytes, ct, tail, lane);                      \
   }
   // Half-tile loop.  Every wave runs the same number of iterations (the longest group's), so the barriers match.
   // A group's leading full halves take the copy of the code without masking; what is left -- at most the one
@@ -639,15 +645,17 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
     const int r = wave >> 1;  // row-block of this wave inside the workgroup
     const int* mine = plan + (1 + r) * p.nKt;
     const int n_mine = uniform_load(plan_cnt, 1 + r);
-    const int n_iter = 2 * max(max(uniform_load(plan_cnt, 1), uniform_load(plan_cnt, 2)),
-                               max(uniform_load(plan_cnt, 3), uniform_load(plan_cnt, 4)));
+    int n_longest = 0;  // every wave runs as many iterations as the longest list needs, so the barriers match
+#pragma unroll
+    for (int rr = 0; rr < kSparseRows; ++rr) n_longest = max(n_longest, uniform_load(plan_cnt, 1 + rr));
+    const int n_iter = 2 * n_longest;
     constexpr int kKHalf = kKBytes / 2, kVHalf = kVTileBytes / 2;
     // this wave copies half of its pair's K half (and V half): K images are 1 KiB x (8 bf16 | 4 fp8) per half
     auto dma_half = [&](int it, int stage) {
       const int tile = uniform_load(mine, it >> 1);
       const int kb = it & 1;
       const char* g = p.kv + (int64_t)bh * p.kv_bh_stride + (int64_t)tile * p.kv_tile_stride;
-      char* d = lds_raw + (stage * 4 + r) * kHalfBytes;
+      char* d = lds_raw + (stage * kSparseRows + r) * kHalfBytes;
       const int sub = wave & 1;
 #pragma unroll
       for (int i = 0; i < kKHalf / 2048; ++i)
@@ -658,15 +666,21 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == kShortWaves ? 3 : 1)) void at
                   d + kKHalf + (sub * (kVHalf / 2048) + i) * 1024);
     };
     __syncthreads();  // every wave is done with the phase-1 ring
-    if (n_mine > 0) dma_half(0, 0);
+    // kStages2 - 1 half tiles ahead: half tile `it` lives in stage it % kStages2
+#pragma unroll
+    for (int a = 0; a < kStages2 - 1; ++a)
+      if (a < 2 * n_mine) dma_half(a, a);
+    int st2 = 0, st2_free = kStages2 - 1;  // stage of half tile `it`, and the one the newest copy goes to
 #define PKH3_HALF_LOOP(STATIC)                                                                          \
   for (int it = 0; it < n_iter; ++it) {                                                                 \
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
     __syncthreads();                                                                                    \
-    if (it + 1 < 2 * n_mine) dma_half(it + 1, (it + 1) & 1);                                            \
+    if (it + kStages2 - 1 < 2 * n_mine) dma_half(it + kStages2 - 1, st2_free);                          \
+    const char* hbuf = lds_raw + (st2 * kSparseRows + r) * kHalfBytes;                                  \
+    st2_free = st2;                                                                                     \
+    st2 = st2 == kStages2 - 1 ? 0 : st2 + 1;                                                            \
     if (it >= 2 * n_mine) continue; /* wave-uniform: this row-block has run out of tiles */             \
     const int tile = uniform_load(mine, it >> 1);                                                       \
-    const char* hbuf = lds_raw + ((it & 1) * 4 + r) * kHalfBytes;                                       \
     qk_half<FP8>(w, hbuf, hbuf + kKHalf, lane);                                                         \
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
     const int lim = (tail && tile == nkt - 1) ? tail - 32 * (it & 1) : 32;                              \
@@ -763,10 +777,10 @@ hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Block-sparse plan.  For each workgroup (4 consecutive 64-query row-blocks) five ascending tile lists, each
-// `nKt` ints apart: [0] the key tiles every one of its row-blocks keeps (walked by all 8 waves together),
-// [1+r] the tiles row-block r keeps that are not in [0] (walked by that row-block's wave pair).  One
-// workgroup per query tile merges the four CSR rows through an LDS mask array, key tiles in chunks.
+// Block-sparse plan.  For each workgroup (kSparseRows consecutive 64-query row-blocks) 1 + kSparseRows ascending
+// tile lists, each `nKt` ints apart: [0] the key tiles every one of its row-blocks keeps (walked by all its waves
+// together), [1+r] the tiles row-block r keeps that are not in [0] (walked by that row-block's wave pair).  One
+// workgroup per attention workgroup merges the CSR rows through an LDS mask array, key tiles in chunks.
 constexpr int kPlanChunk = 8192;
 
 __global__ __launch_bounds__(256) void sparse_plan_kernel(const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
@@ -774,17 +788,17 @@ __global__ __launch_bounds__(256) void sparse_plan_kernel(const int* __restrict_
                                                           int* __restrict__ plan_cnt) {
   __shared__ unsigned char mask[kPlanChunk];
   __shared__ int wave_tot[4];
-  __shared__ int carry[5];
+  __shared__ int carry[kSparseLists];
   const int qt = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int* out = plan + (int64_t)qt * plan_stride;
-  const int rows_here = min(4, nRow64 - qt * 4);
+  const int rows_here = max(0, min(kSparseRows, nRow64 - qt * kSparseRows));
   const int full = (1 << rows_here) - 1;
-  if (tid < 5) carry[tid] = 0;
+  if (tid < kSparseLists) carry[tid] = 0;
   for (int base = 0; base < nKt; base += kPlanChunk) {
     for (int i = tid; i < kPlanChunk; i += 256) mask[i] = 0;
     __syncthreads();
     for (int r = 0; r < rows_here; ++r) {
-      const int row = qt * 4 + r;
+      const int row = qt * kSparseRows + r;
       const int beg = row_ptr[row], end = row_ptr[row + 1];
       for (int j = beg + tid; j < end; j += 256) {
         const int col = col_idx[j] - base;
@@ -793,7 +807,7 @@ __global__ __launch_bounds__(256) void sparse_plan_kernel(const int* __restrict_
       }
       __syncthreads();
     }
-    for (int list = 0; list < 5; ++list) {
+    for (int list = 0; list < kSparseLists; ++list) {
       for (int c0 = 0; c0 < kPlanChunk && base + c0 < nKt; c0 += 256) {
         const int col = c0 + tid;
         const int mk = (base + col < nKt) ? mask[col] : 0;
@@ -811,12 +825,12 @@ __global__ __launch_bounds__(256) void sparse_plan_kernel(const int* __restrict_
       }
     }
   }
-  if (tid < 5) plan_cnt[qt * 5 + tid] = carry[tid];
+  if (tid < kSparseLists) plan_cnt[qt * kSparseLists + tid] = carry[tid];
 }
 
 hipError_t launch_sparse_plan(const int* row_ptr, const int* col_idx, int nRow64, int nQ64, int nKt, int* plan,
                               int plan_stride, int* plan_cnt, hipStream_t st) {
-  hipLaunchKernelGGL(sparse_plan_kernel, dim3(nQ64 / 4), dim3(256), 0, st, row_ptr, col_idx, nRow64, nKt, plan, plan_stride,
+  hipLaunchKernelGGL(sparse_plan_kernel, dim3(nQ64 / kSparseRows), dim3(256), 0, st, row_ptr, col_idx, nRow64, nKt, plan, plan_stride,
                      plan_cnt);
   return hipGetLastError();
 }

@@ -8,6 +8,11 @@
 
 namespace pkh3 {
 
+// Block-sparse work split: a workgroup covers kSparseRows consecutive 64-query row-blocks (a wave pair each) and its
+// plan holds 1 + kSparseRows tile lists (the tiles all its row-blocks keep, then one list per row-block).
+constexpr int kSparseRows = 2;
+constexpr int kSparseLists = 1 + kSparseRows;
+
 // Where each intermediate lives inside the caller's workspace (byte offsets, 256-aligned).
 struct WsPlan {
   int nQ64;      // 64-query blocks, padded to a multiple of 4 (one workgroup = 4 waves x 64 queries)
@@ -66,9 +71,9 @@ struct FwdParams {
   int B, H, Sq, Sk;
   int nQ64, nKt;
   float c;                  // softmax_scale * log2(e)
-  const int* plan;          // block-sparse: per query tile (256 queries) five tile lists nKt ints apart, or null
-  const int* plan_cnt;      // [nQ64/4][5] entries per list
-  int plan_stride;          // ints between consecutive query tiles' lists (5 * nKt)
+  const int* plan;          // block-sparse: per workgroup kSparseLists tile lists nKt ints apart, or null
+  const int* plan_cnt;      // [nQ64/kSparseRows][kSparseLists] entries per list
+  int plan_stride;          // ints between consecutive workgroups' lists (kSparseLists * nKt)
   const float* kscale;      // [B*H, nKt] fp8 dequantisation scales of the K tiles
   const float* kmax;        // [B*H] largest K' row norm
   int fp8;

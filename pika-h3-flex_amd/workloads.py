@@ -96,6 +96,56 @@ def plumbing_inputs(*, heads: int = 4, seq: int = 1024, seed: int = 0, device="c
     return AttnInputs(q, k, v, None, None, "plumbing")
 
 
+@dataclass
+class BlockInputs:
+    """The attention half of one DiT block at a self-attention configuration: hidden states, the four projections
+    with their LoRA adapters (rank 128 on ``to_q, to_k, to_v, to_out.0``, src/pika_h3/core/loader.py:9), AdaLN
+    tables gathered per row by ``row_index`` (three timestep groups), and the position grid."""
+
+    x: torch.Tensor                    # [S, C] bf16
+    linears: dict                      # "q" | "k" | "v" | "out" -> dict(weight, bias, lora_a, lora_b, lora_scale)
+    shift: torch.Tensor                # [T, C] bf16
+    scale: torch.Tensor
+    gate: torch.Tensor
+    row_index: torch.Tensor            # [S] int32
+    position_ids: torch.Tensor         # [S, 3] float64
+    heads: int
+    name: str
+
+    @property
+    def attention_flops(self) -> float:
+        S = self.x.shape[0]
+        return 4.0 * S * S * HEAD_DIM * self.heads
+
+    @property
+    def projection_flops(self) -> float:
+        """2*S*C*N over the four projections plus the adapters' two rank-128 products each."""
+        S, C = self.x.shape
+        r = next(iter(self.linears.values()))["lora_a"].shape[0]
+        return 4 * (2.0 * S * C * C) + 4 * (2.0 * S * C * r + 2.0 * S * r * C)
+
+
+def block_inputs(*, frames: int, rows_h: int, rows_w: int, heads: int = 24, lora_rank: int = 128, lora_alpha: int = 64,
+                 groups: int = 3, seed: int = 0, device="cuda", name: str = "block") -> BlockInputs:
+    gen = torch.Generator().manual_seed(int(seed))
+    C = heads * HEAD_DIM
+    pos = video_position_ids(frames, rows_h, rows_w)
+    S = pos.shape[0]
+    x = _randn((S, C), gen, device)
+    lin = {}
+    for n in ("q", "k", "v", "out"):
+        lin[n] = dict(
+            weight=_randn((C, C), gen, device, std=0.02),
+            bias=(torch.randn((C,), generator=gen) * 0.02).to(device),
+            lora_a=_randn((lora_rank, C), gen, device, std=0.02),
+            lora_b=_randn((C, lora_rank), gen, device, std=0.02),
+            lora_scale=float(lora_alpha) / float(lora_rank),
+        )
+    shift, scale, gate = (_randn((groups, C), gen, device, std=0.2) for _ in range(3))
+    row_index = (torch.arange(S) * groups // S).to(torch.int32).to(device)
+    return BlockInputs(x, lin, shift, scale, gate, row_index, pos.to(device), heads, name)
+
+
 # The benchmark configurations by name.
 CONFIGS = {
     "plumbing": dict(kind="plumbing", heads=4, seq=1024),
