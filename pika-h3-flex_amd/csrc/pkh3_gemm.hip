@@ -45,22 +45,28 @@ __device__ __forceinline__ void gemm_dma16(const char* g, unsigned lane_off, cha
 // lane's row in the layout of norm_rope_row, i.e. index 16*db + i of its x[64] (see pack_rows_kernel for the
 // weight-row permutation that makes it so).
 
-template <int EPI>
+// WAVES = 8 (the form that ships): wave tile 128 features x 64 tokens, two waves per SIMD, accumulators in 128 VGPRs.
+// WAVES = 4 (wave tile 128 x 128, one wave per SIMD, 256 accumulator registers, half the LDS reads per MFMA) compiles
+// and passes the same tests but measured four times slower: with more than 256 registers the compiler moves
+// accumulators between the two register files inside the loop.
+template <int EPI, int WAVES>
 __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget& tg, int m_tile, int n_tile_in_target,
                                           char* lds_raw) {
+  constexpr int TB = 16 / WAVES;                     // 32-token blocks per wave
+  constexpr int PP = 32 / WAVES;                     // 1 KiB pieces of a chunk each wave copies
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int hh = lane >> 5, r = lane & 31;
-  const int fh = wave & 1, tq = wave >> 1;
+  const int fh = wave & 1, tq = wave >> 1;           // feature half (one head), token slice
   const int head = n_tile_in_target * 2 + fh;        // 128-feature head inside the target
   const bool head_live = head * 128 < tg.n;
   const int nk1 = p.nk1, nk = p.nk1 + tg.nk2;
   const unsigned lane_off = lane * 16;
 
-  // this wave's four 1 KiB pieces of every chunk: pieces 4*wave..4*wave+3 of [8 weight blocks x 2 | 8 token blocks x 2]
-  const int piece0 = wave * 4;
+  // this wave's 1 KiB pieces of every chunk: pieces PP*wave.. of [8 weight blocks x 2 k-steps | 8 token blocks x 2]
+  const int piece0 = wave * PP;
   const bool w_side = piece0 < 16;
-  const int blk0 = (piece0 & 15) >> 1;               // first of the two 32-row blocks this wave copies
+  const int blk0 = (piece0 & 15) >> 1;               // first of the 32-row blocks this wave copies
   const char* seg1 = w_side ? tg.w_img + (int64_t)(n_tile_in_target * 8 + blk0) * tg.w_blk_stride
                             : p.a_img + (int64_t)(m_tile * 8 + blk0) * p.a_blk_stride;
   const int64_t seg1_step = w_side ? tg.w_blk_stride : p.a_blk_stride;
@@ -73,15 +79,22 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
     const char* g = first ? seg1 + (int64_t)kc * 2048 : seg2 + (int64_t)(kc - nk1) * 2048;
     const int64_t step = first ? seg1_step : seg2_step;
     // two consecutive k-step images of one block are contiguous (2 KiB); the next block is `step` bytes on
-    gemm_dma16(g, lane_off, d);
-    gemm_dma16(g + 1024, lane_off, d + 1024);
-    gemm_dma16(g + step, lane_off, d + 2048);
-    gemm_dma16(g + step + 1024, lane_off, d + 3072);
+#pragma unroll
+    for (int b = 0; b < PP / 2; ++b) {
+      gemm_dma16(g + b * step, lane_off, d + b * 2048);
+      gemm_dma16(g + b * step + 1024, lane_off, d + b * 2048 + 1024);
+    }
+  };
+  // waits until at most `chunks` of this wave's newest chunk copies are still in flight
+  auto wait_dma = [&](int chunks) {
+    if (chunks >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PP) : "memory");
+    else if (chunks == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PP) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
 
-  f32x16 acc[2][4];
+  f32x16 acc[TB][4];
 #pragma unroll
-  for (int t2 = 0; t2 < 2; ++t2)
+  for (int t2 = 0; t2 < TB; ++t2)
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -93,27 +106,25 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
   // read at the tail of this iteration and no wave starts a chunk by waiting for LDS.
   const int n_pre = nk < 3 ? nk : 3;
   for (int c = 0; c < n_pre; ++c) dma(c, c);
-  if (n_pre == 3) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  else if (n_pre == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  wait_dma(n_pre - 1);
   __syncthreads();
   const int w_off = (fh * 4) * 2048 + lane * 16;            // weight blocks fh*4..+3 of a slot
-  const int a_off = 16384 + (tq * 2) * 2048 + lane * 16;    // token blocks tq*2, +1
-  bf16x8 wf[2][4], xf[2][2];
-  auto read_frags = [&](int slot, int ks, bf16x8 (&w4)[4], bf16x8 (&x2)[2]) {
+  const int a_off = 16384 + (tq * TB) * 2048 + lane * 16;   // this wave's token blocks
+  bf16x8 wf[2][4], xf[2][TB];
+  auto read_frags = [&](int slot, int ks, bf16x8 (&w4)[4], bf16x8 (&xt)[TB]) {
     const char* base = lds_raw + slot * kGemmStageBytes + ks * 1024;
 #pragma unroll
     for (int db = 0; db < 4; ++db) w4[db] = *(const bf16x8*)(base + w_off + db * 2048);
 #pragma unroll
-    for (int t2 = 0; t2 < 2; ++t2) x2[t2] = *(const bf16x8*)(base + a_off + t2 * 2048);
+    for (int t2 = 0; t2 < TB; ++t2) xt[t2] = *(const bf16x8*)(base + a_off + t2 * 2048);
   };
-  auto mfma8 = [&](const bf16x8 (&w4)[4], const bf16x8 (&x2)[2]) {
+  auto mfmas = [&](const bf16x8 (&w4)[4], const bf16x8 (&xt)[TB]) {
 #pragma unroll
-    for (int t2 = 0; t2 < 2; ++t2)
+    for (int t2 = 0; t2 < TB; ++t2)
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
-        if constexpr (EPI == kEpiVImg) acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x2[t2], w4[db], acc[t2][db], 0, 0, 0);
-        else acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w4[db], x2[t2], acc[t2][db], 0, 0, 0);
+        if constexpr (EPI == kEpiVImg) acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xt[t2], w4[db], acc[t2][db], 0, 0, 0);
+        else acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w4[db], xt[t2], acc[t2][db], 0, 0, 0);
       }
   };
   if (head_live) read_frags(0, 0, wf[0], xf[0]);
@@ -121,150 +132,154 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
   for (int kc = 0; kc < nk; ++kc) {
     if (kc + 1 < nk) {
       // chunk kc+1 has landed (this wave's pieces; the barrier covers the others'); only chunk kc+2's copies may be pending
-      if (kc + 2 < nk) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (kc + 2 < nk) wait_dma(1);
+      else wait_dma(0);
       __syncthreads();
       if (kc + 3 < nk) dma(kc + 3, (slot + 3) & 3);
     }
     const int next = (slot + 1) & 3;
     if (head_live) {  // wave-uniform: a head past the end of the target only copies and synchronises
       read_frags(slot, 1, wf[1], xf[1]);
-      mfma8(wf[0], xf[0]);
+      mfmas(wf[0], xf[0]);
       if (kc + 1 < nk) read_frags(next, 0, wf[0], xf[0]);
-      mfma8(wf[1], xf[1]);
+      mfmas(wf[1], xf[1]);
     }
     slot = next;
   }
   // let the last MFMA retire before anything the compiler places after the loop reads the accumulators
-  asm volatile("s_nop 15\n\ts_nop 15"
-               : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]), "+v"(acc[1][1]),
-                 "+v"(acc[1][2]), "+v"(acc[1][3])::"memory");
+#pragma unroll
+  for (int t2 = 0; t2 < TB; ++t2)
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc[t2][0]), "+v"(acc[t2][1]), "+v"(acc[t2][2]), "+v"(acc[t2][3])::"memory");
   if (!head_live) return;
 
-  const int tok0 = m_tile * kGemmTile + tq * 64;     // first of this wave's 64 tokens = one K/V tile
-  const int tile = m_tile * 4 + tq;
-  if (tok0 >= p.M) return;                           // a tile past the last token: nothing to write
   const float* bias = tg.bias ? tg.bias + head * 128 : nullptr;
+  // the wave's token blocks, two at a time: one 64-token K/V tile per pair
+#pragma unroll
+  for (int tp = 0; tp < TB / 2; ++tp) {
+    const int tok0 = m_tile * kGemmTile + tq * (32 * TB) + tp * 64;
+    const int tile = m_tile * 4 + tq * (TB / 2) + tp;
+    if (tok0 >= p.M) break;                          // tiles past the last token: nothing to write
 
-  if constexpr (EPI == kEpiVImg) {
-    // lane = feature 32*db + r of the head, registers = tokens: exactly the V image rows
-    char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
-#pragma unroll
-    for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-      for (int b2 = 0; b2 < 2; ++b2)
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const float bv = bias ? bias[32 * db + r] : 0.f;
-          bf16x8 img;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int token = tok0 + 32 * t2 + 8 * (2 * b2 + j / 4) + 4 * hh + (j % 4);
-            img[j] = token < p.M ? (__bf16)(acc[t2][db][8 * b2 + j] + bv) : (__bf16)0.0f;
-          }
-          *(bf16x8*)(rec + (((t2 * 2 + b2) * 4 + db) * 64 + lane) * 16) = img;
-        }
-    return;
-  } else {
-    // lane = token, its 64 accumulator values per token block = head-dim elements 16*ks + 8*hh + j in x[ks*8 + j]
-    float x[2][64];
-#pragma unroll
-    for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) x[t2][16 * db + i] = acc[t2][db][i] * tg.out_scale;   // x index = ks*8 + j
-    if (bias) {
+    if constexpr (EPI == kEpiVImg) {
+      // lane = feature 32*db + r of the head, registers = tokens: exactly the V image rows
+      char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
 #pragma unroll
       for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-          const f32x4 b0 = *(const f32x4*)(bias + 16 * ks + 8 * hh), b1 = *(const f32x4*)(bias + 16 * ks + 8 * hh + 4);
+        for (int b2 = 0; b2 < 2; ++b2)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            x[t2][ks * 8 + j] += b0[j];
-            x[t2][ks * 8 + 4 + j] += b1[j];
+          for (int db = 0; db < 4; ++db) {
+            const float bv = bias ? bias[32 * db + r] : 0.f;
+            bf16x8 img;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const int token = tok0 + 32 * t2 + 8 * (2 * b2 + j / 4) + 4 * hh + (j % 4);
+              img[j] = token < p.M ? (__bf16)(acc[2 * tp + t2][db][8 * b2 + j] + bv) : (__bf16)0.0f;
+            }
+            *(bf16x8*)(rec + (((t2 * 2 + b2) * 4 + db) * 64 + lane) * 16) = img;
           }
-        }
-    }
-    if constexpr (EPI == kEpiKImg) {
-      const RowTransform tf{tg.norm_w, tg.norm_eps, tg.rope_mode, tg.cos_t, tg.sin_t};
-      float nmax = 0.f, amax = 0.f;
+    } else {
+      // lane = token, its 64 accumulator values per token block = head-dim elements 16*ks + 8*hh + j in x[ks*8 + j]
+      float x[2][64];
 #pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) {
-        const int token = tok0 + 32 * t2 + r;
-        const bool valid = token < p.M;
-        if (!valid) {
+      for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-          for (int i = 0; i < 64; ++i) x[t2][i] = 0.f;
-        }
-        norm_rope_row(x[t2], tf, valid ? token : 0, valid, hh);
-        float ssq = 0.f;
+        for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int i = 0; i < 64; ++i) {
-          ssq += x[t2][i] * x[t2][i];
-          amax = fmaxf(amax, fabsf(x[t2][i]));
-        }
-        nmax = fmaxf(nmax, ssq + xhalf(ssq));
-      }
-      if (tg.norm_max) {
-        nmax = sqrtf(wave_max(nmax));
-        if (lane == 0) atomicMax(tg.norm_max + head, __float_as_uint(nmax));
-      }
-      char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
-      if (!tg.fp8) {
+          for (int i = 0; i < 16; ++i) x[t2][16 * db + i] = acc[2 * tp + t2][db][i] * tg.out_scale;   // x index = ks*8 + j
+      if (bias) {
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
           for (int ks = 0; ks < 8; ++ks) {
-            bf16x8 t;
+            const f32x4 b0 = *(const f32x4*)(bias + 16 * ks + 8 * hh), b1 = *(const f32x4*)(bias + 16 * ks + 8 * hh + 4);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[t2][ks * 8 + j];
-            *(bf16x8*)(rec + t2 * tg.out_sub_stride + (ks * 64 + lane) * 16) = t;
+            for (int j = 0; j < 4; ++j) {
+              x[t2][ks * 8 + j] += b0[j];
+              x[t2][ks * 8 + 4 + j] += b1[j];
+            }
           }
-      } else {
-        amax = wave_max(amax);
-        const float scale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
-        const float inv = 1.0f / scale;
-        if (lane == 0) tg.scale_out[(int64_t)head * tg.scale_head_stride + tile] = scale;
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-          for (int c = 0; c < 4; ++c)
-            *(i32x4*)(rec + t2 * tg.out_sub_stride + (c * 64 + lane) * 16) = quant_fp8_chunk(x[t2], c, inv);
       }
-    } else {
-      // row-major bf16 rows: y = residual + gate[row_index] * (acc*scale + bias); 16-byte pieces per lane
+      if constexpr (EPI == kEpiKImg) {
+        const RowTransform tf{tg.norm_w, tg.norm_eps, tg.rope_mode, tg.cos_t, tg.sin_t};
+        float nmax = 0.f, amax = 0.f;
 #pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) {
-        const int token = tok0 + 32 * t2 + r;
-        if (token >= p.M) continue;
-        __bf16* orow = (__bf16*)tg.out + (int64_t)token * tg.out_row_stride + (int64_t)head * tg.out_head_elems;
-        const __bf16* res = tg.residual ? (const __bf16*)tg.residual + (int64_t)token * tg.res_row_stride + head * 128 : nullptr;
-        const __bf16* gate = tg.gate ? (const __bf16*)tg.gate + (int64_t)(tg.row_index ? tg.row_index[token] : 0) * tg.gate_row_stride + head * 128
-                                     : nullptr;
+        for (int t2 = 0; t2 < 2; ++t2) {
+          const int token = tok0 + 32 * t2 + r;
+          const bool valid = token < p.M;
+          if (!valid) {
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-          const int d0 = 16 * ks + 8 * hh;
-          bf16x8 o;
-          bf16x8 gv, rv;
-          if (gate) gv = *(const bf16x8*)(gate + d0);
-          if (res) rv = *(const bf16x8*)(res + d0);
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            float v = x[t2][ks * 8 + j];
-            if (gate) v *= (float)gv[j];
-            if (res) v += (float)rv[j];
-            o[j] = (__bf16)v;
+            for (int i = 0; i < 64; ++i) x[t2][i] = 0.f;
           }
-          *(bf16x8*)(orow + d0) = o;
+          norm_rope_row(x[t2], tf, valid ? token : 0, valid, hh);
+          float ssq = 0.f;
+#pragma unroll
+          for (int i = 0; i < 64; ++i) {
+            ssq += x[t2][i] * x[t2][i];
+            amax = fmaxf(amax, fabsf(x[t2][i]));
+          }
+          nmax = fmaxf(nmax, ssq + xhalf(ssq));
+        }
+        if (tg.norm_max) {
+          nmax = sqrtf(wave_max(nmax));
+          if (lane == 0) atomicMax(tg.norm_max + head, __float_as_uint(nmax));
+        }
+        char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
+        if (!tg.fp8) {
+#pragma unroll
+          for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+              bf16x8 t;
+#pragma unroll
+              for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[t2][ks * 8 + j];
+              *(bf16x8*)(rec + t2 * tg.out_sub_stride + (ks * 64 + lane) * 16) = t;
+            }
+        } else {
+          amax = wave_max(amax);
+          const float scale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
+          const float inv = 1.0f / scale;
+          if (lane == 0) tg.scale_out[(int64_t)head * tg.scale_head_stride + tile] = scale;
+#pragma unroll
+          for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+              *(i32x4*)(rec + t2 * tg.out_sub_stride + (c * 64 + lane) * 16) = quant_fp8_chunk(x[t2], c, inv);
+        }
+      } else {
+        // row-major bf16 rows: y = residual + gate[row_index] * (acc*scale + bias); 16-byte pieces per lane
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+          const int token = tok0 + 32 * t2 + r;
+          if (token >= p.M) continue;
+          __bf16* orow = (__bf16*)tg.out + (int64_t)token * tg.out_row_stride + (int64_t)head * tg.out_head_elems;
+          const __bf16* res = tg.residual ? (const __bf16*)tg.residual + (int64_t)token * tg.res_row_stride + head * 128 : nullptr;
+          const __bf16* gate = tg.gate ? (const __bf16*)tg.gate + (int64_t)(tg.row_index ? tg.row_index[token] : 0) * tg.gate_row_stride + head * 128
+                                       : nullptr;
+#pragma unroll
+          for (int ks = 0; ks < 8; ++ks) {
+            const int d0 = 16 * ks + 8 * hh;
+            bf16x8 o;
+            bf16x8 gv, rv;
+            if (gate) gv = *(const bf16x8*)(gate + d0);
+            if (res) rv = *(const bf16x8*)(res + d0);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              float v = x[t2][ks * 8 + j];
+              if (gate) v *= (float)gv[j];
+              if (res) v += (float)rv[j];
+              o[j] = (__bf16)v;
+            }
+            *(bf16x8*)(orow + d0) = o;
+          }
         }
       }
     }
   }
 }
 
-__global__ __launch_bounds__(64 * kGemmWaves, 1) void gemm_kernel(GemmParams p) {
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 1) void gemm_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(1024))) char lds_raw[kGemmRing * kGemmStageBytes];
   // Workgroups go to the 8 XCDs round-robin; each XCD takes one contiguous run of the tile order below, in which 32
   // consecutive tiles (the workgroups the 32 CUs behind one L2 run together) form a block of 4 token tiles x 8
@@ -289,15 +304,15 @@ __global__ __launch_bounds__(64 * kGemmWaves, 1) void gemm_kernel(GemmParams p) 
   while (t + 1 < p.n_targets && n_tile >= p.tg[t].n_tiles) { n_tile -= p.tg[t].n_tiles; ++t; }
   const GemmTarget& tg = p.tg[t];
   switch (tg.epi) {
-    case kEpiRows: gemm_tile<kEpiRows>(p, tg, m_tile, n_tile, lds_raw); break;
-    case kEpiKImg: gemm_tile<kEpiKImg>(p, tg, m_tile, n_tile, lds_raw); break;
-    default: gemm_tile<kEpiVImg>(p, tg, m_tile, n_tile, lds_raw); break;
+    case kEpiRows: gemm_tile<kEpiRows, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
+    case kEpiKImg: gemm_tile<kEpiKImg, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
+    default: gemm_tile<kEpiVImg, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
   }
 }
 
 hipError_t launch_gemm(const GemmParams& p, hipStream_t st) {
   const int total = p.m_tiles * p.n_tiles;
-  hipLaunchKernelGGL(gemm_kernel, dim3((total + 7) / 8 * 8), dim3(64 * kGemmWaves), 0, st, p);
+  hipLaunchKernelGGL(gemm_kernel<kGemmWaves>, dim3((total + 7) / 8 * 8), dim3(64 * kGemmWaves), 0, st, p);
   return hipGetLastError();
 }
 

@@ -10,7 +10,7 @@ namespace pkh3 {
 
 // Block-sparse work split: a workgroup covers kSparseRows consecutive 64-query row-blocks (a wave pair each) and its
 // plan holds 1 + kSparseRows tile lists (the tiles all its row-blocks keep, then one list per row-block).
-constexpr int kSparseRows = 2;
+constexpr int kSparseRows = 4;
 constexpr int kSparseLists = 1 + kSparseRows;
 
 // Where each intermediate lives inside the caller's workspace (byte offsets, 256-aligned).

@@ -186,3 +186,131 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, f"{f} mentions the oracle"
+
+
+# ---- projection entry points: host-side validation, no GPU ---------------------------------------------------
+def test_packed_bytes_host_only(lib):
+    assert lib.pkh3_packed_bytes(1, 32) == 256 * 32 * 2                  # rows padded to 256
+    assert lib.pkh3_packed_bytes(48360, 3072) == 48384 * 3072 * 2
+    assert lib.pkh3_packed_bytes(256, 4096) == 256 * 4096 * 2
+    for rows, k in ((0, 64), (8, 0), (8, 48), (8, 4128), (-1, 64)):
+        assert lib.pkh3_packed_bytes(rows, k) == 0
+
+
+def test_pack_and_modulate_argument_errors(lib):
+    x, out = 0x10000, 0x200000
+    assert lib.pkh3_pack_rows(None, 64, 8, 64, out, None) == _lib.PKH3_ENULL
+    assert lib.pkh3_pack_rows(x, 64, 8, 64, None, None) == _lib.PKH3_ENULL
+    assert lib.pkh3_pack_rows(x + 2, 64, 8, 64, out, None) == _lib.PKH3_EALIGN
+    assert lib.pkh3_pack_rows(x, 64, 8, 64, out + 16, None) == _lib.PKH3_EALIGN      # destination: 256-byte aligned
+    assert lib.pkh3_pack_rows(x, 64, 0, 64, out, None) == _lib.PKH3_ESHAPE
+    assert lib.pkh3_pack_rows(x, 64, 8, 48, out, None) == _lib.PKH3_ESHAPE           # K multiple of 32
+    assert lib.pkh3_pack_rows(x, 8192, 8, 8192, out, None) == _lib.PKH3_ESHAPE       # K <= 4096
+    assert lib.pkh3_pack_rows(x, 32, 8, 64, out, None) == _lib.PKH3_ESTRIDE          # stride < K
+    assert lib.pkh3_pack_rows(x, 68, 8, 64, out, None) == _lib.PKH3_ESTRIDE          # stride not a multiple of 8
+    assert lib.pkh3_pack_weight(x, 64, 100, 64, 1, out, None) == _lib.PKH3_ESHAPE    # whole 128-feature heads
+    assert b"128" in lib.pkh3_last_error()
+    mod = lib.pkh3_adaln_modulate
+    assert mod(x, 64, 8, 64, 7, 1e-6, None, None, 0, None, out, None) == _lib.PKH3_EARG               # norm kind
+    assert mod(x, 64, 8, 64, _lib.NORM_LAYER, float("nan"), None, None, 0, None, out, None) == _lib.PKH3_EARG
+    assert mod(x, 64, 8, 64, _lib.NORM_NONE, 0.0, 0x30000, None, 64, None, out, None) == _lib.PKH3_EUNSUPPORTED
+    assert mod(x, 64, 8, 64, _lib.NORM_LAYER, 1e-6, 0x30002, None, 64, None, out, None) == _lib.PKH3_EALIGN
+    assert mod(x, 64, 8, 64, _lib.NORM_LAYER, 1e-6, 0x30000, None, 32, None, out, None) == _lib.PKH3_ESTRIDE
+
+
+def _qkv_args():
+    a = _valid_args()
+    a.B, a.H, a.Sq, a.Sk = 1, 2, 64, 64
+    p = _lib.QkvArgs()
+    p.x_img, p.S, p.K = 0x400000, 64, 256
+    for lin in (p.q, p.k, p.v):
+        lin.w_img = 0x500000
+    return p, a
+
+
+def test_qkv_proj_argument_errors(lib):
+    p, a = _qkv_args()
+    assert lib.pkh3_qkv_proj(None, C.byref(a), None) == _lib.PKH3_ENULL
+    assert lib.pkh3_qkv_proj(C.byref(p), None, None) == _lib.PKH3_ENULL
+    p, a = _qkv_args(); a.k = a.v = 0                                    # K and V inputs are not needed
+    a.B = 2
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_EUNSUPPORTED
+    p, a = _qkv_args(); a.key_mask = 0x40000
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_EUNSUPPORTED
+    p, a = _qkv_args(); a.Sk = 128
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_EUNSUPPORTED
+    p, a = _qkv_args(); p.S = 65
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_ESHAPE
+    p, a = _qkv_args(); p.K = 100
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_ESHAPE
+    p, a = _qkv_args(); p.x_img = 0
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_ENULL
+    p, a = _qkv_args(); p.k.w_img = 0
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_ENULL
+    p, a = _qkv_args(); p.v.lora_a_img = 0x600000                        # A without B
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_ENULL
+    p, a = _qkv_args(); p.v.lora_a_img = p.v.lora_b_img = 0x600000       # adapter without its scratch
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_EWORKSPACE
+    p, a = _qkv_args(); a.workspace_bytes = 1024
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_EWORKSPACE
+    # the attention call on prepared K/V: k and v may be NULL, but the shape restrictions stay
+    p, a = _qkv_args(); a.k = a.v = 0
+    assert lib.pkh3_attn_fwd(C.byref(a), None) == _lib.PKH3_ENULL
+    a.flags = _lib.FLAG_KV_PREPARED; a.B = 2
+    assert lib.pkh3_attn_fwd(C.byref(a), None) == _lib.PKH3_EUNSUPPORTED
+    a.B = 1
+    assert lib.pkh3_attn_fwd_noalloc(C.byref(a), None) == _lib.PKH3_EUNSUPPORTED
+
+
+def test_out_proj_argument_errors(lib):
+    def ok():
+        o = _lib.OutArgs()
+        o.o_img, o.S, o.K, o.N = 0x400000, 64, 256, 256
+        o.proj.w_img = 0x500000
+        o.y, o.y_stride = 0x700000, 256
+        return o
+    assert lib.pkh3_out_proj(None, None) == _lib.PKH3_ENULL
+    for mutate, code in [
+        (lambda o: setattr(o, "S", 0), _lib.PKH3_ESHAPE), (lambda o: setattr(o, "K", 40), _lib.PKH3_ESHAPE),
+        (lambda o: setattr(o, "N", 100), _lib.PKH3_ESHAPE), (lambda o: setattr(o, "o_img", 0), _lib.PKH3_ENULL),
+        (lambda o: setattr(o, "y", 0), _lib.PKH3_ENULL), (lambda o: setattr(o, "y_stride", 128), _lib.PKH3_ESTRIDE),
+        (lambda o: (setattr(o, "gate", 0x800000), setattr(o, "gate_stride", 100)), _lib.PKH3_ESTRIDE),
+        (lambda o: (setattr(o, "residual", 0x800004), setattr(o, "residual_stride", 256)), _lib.PKH3_ESTRIDE),
+        (lambda o: setattr(o.proj, "w_img", 0), _lib.PKH3_ENULL),
+        (lambda o: (setattr(o.proj, "lora_a_img", 0x600000), setattr(o.proj, "lora_b_img", 0x600000)), _lib.PKH3_EWORKSPACE),
+    ]:
+        o = ok()
+        mutate(o)
+        assert lib.pkh3_out_proj(C.byref(o), None) == code, lib.pkh3_last_error()
+
+
+def test_projection_struct_layouts_match_header():
+    header = open(os.path.join(ROOT, "include", "pkh3_attn.h")).read()
+    for name, mirror in (("pkh3_linear", _lib.Linear), ("pkh3_qkv_args", _lib.QkvArgs), ("pkh3_out_args", _lib.OutArgs)):
+        body = header[header.index("typedef struct %s {" % name): header.index("} %s;" % name)]
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        names = []
+        for decl in body.split("{", 1)[1].split(";"):
+            decl = decl.strip()
+            if not decl:
+                continue
+            for part in decl.split(","):
+                names.append(re.findall(r"[A-Za-z_][A-Za-z_0-9]*", part)[-1])
+        assert names == [f[0] for f in mirror._fields_], name
+    assert re.search(r"#define\s+PKH3_LORA_RANK\s+128", header) and _lib.LORA_RANK == 128
+
+
+def test_projection_front_end_refuses_host_tensors():
+    import torch
+
+    from pika_h3_flex_amd import projections as P
+
+    x = torch.zeros((8, 64), dtype=torch.bfloat16)
+    for fn in (P.pack_rows, P.pack_weight, P.adaln_modulate):
+        with pytest.raises(ValueError, match="device memory"):
+            fn(x)
+    with pytest.raises(ValueError, match="bfloat16"):
+        P.pack_rows(x.float())
+    with pytest.raises(ValueError):
+        P.packed_bytes(8, 48)
+    assert P.packed_bytes(300, 64) == 512 * 64 * 2
