@@ -27,9 +27,15 @@ HBM_PEAK_GBS = 8000.0
 # factors from a 1 GiB copy) in earlier profiling runs of the same command, not in this run: (bytes, file that holds
 # the counter values and the commands)
 MEASURED_TRAFFIC = {
-    "480p": (3.96e9, "profiles/attn_fwd_kernel_480p_bf16.md"),
-    "480p-sparse-fp8": (2.12e10, "profiles/attn_fwd_kernel_480p_sparse_fp8.md"),
+    "480p": (4.06e9, "profiles/attn_fwd_kernel_480p_bf16.md"),
+    "480p-fp8": (3.27e9, "profiles/attn_fwd_kernel_480p_fp8.md"),
+    "480p-sparse": (3.158e10, "profiles/attn_fwd_kernel_480p_sparse_bf16.md"),
+    "480p-sparse-fp8": (2.135e10, "profiles/attn_fwd_kernel_480p_sparse_fp8.md"),
+    "768p": (1.366e11, "profiles/attn_fwd_kernel_768p_bf16.md"),
+    "joint": (4.52e9, "profiles/attn_fwd_kernel_joint_bf16.md"),
+    "cross": (6.15e8, "profiles/attn_fwd_kernel_cross_short_key.md"),
 }
+GEMM_TRAFFIC = (6.28e9, "profiles/gemm_kernel_480p_block.md")  # to_q/to_k/to_v launch of the 480p block
 
 
 def host_cpu():
@@ -160,7 +166,7 @@ def bench_block(args, pk, workloads, dev) -> int:
                    "ms_out_projection_with_packing": round(ms_out, 4),
                    "out_projection_tflops": round(flops_out / (ms_out * 1e-3) / 1e12, 2)},
         "roofline": {"bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(gemm_tflops / peak, 4), "traffic": None, "kernel": "gemm_kernel (to_q/to_k/to_v + LoRA, two launches)",
+                     "frac": round(gemm_tflops / peak, 4), "traffic": GEMM_TRAFFIC[0], "traffic_source": GEMM_TRAFFIC[1], "kernel": "gemm_kernel (to_q/to_k/to_v + LoRA, two launches)",
                      "kernel_ms": round(ms_qkv, 4), "flops_per_launch": flops_qkv},
         "cpu_baseline": None,
     }
