@@ -54,6 +54,35 @@ def test_block_sparse_bf16(Sq, Sk, density):
     assert err <= 2e-2 and cos >= 0.9999
 
 
+def test_block_sparse_one_row_private_tile_every_query_block():
+    """One workgroup (256 queries, 1 head) whose first row-block keeps one tile the others do not: the shared walk is
+    a single tile and the row-private walk a single tile of one wave pair.  This is the shape on which a stale 32-row
+    block of the output accumulators was once returned (reads of the accumulators placed right behind the last MFMA
+    of a tile loop, before its result was written back); every 32-query block is therefore checked on its own."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as O
+
+    gen = torch.Generator().manual_seed(1)
+    q, k, v = (_rand((1, 256, 1, D), gen) for _ in range(3))
+    tm = torch.tensor([[1, 0, 0, 1], [1, 0, 0, 0], [1, 0, 0, 0], [1, 0, 0, 0]], dtype=torch.bool)
+    ref = O.reference_layer(q, k, v, tile_map=tm)
+    bm = pk.BlockMask.from_dense(tm, device="cuda")
+    outs = [_call(q, k, v, block_mask=bm) for _ in range(3)]
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+    err = (outs[0].double() - ref).abs()[0, :, 0]
+    per_block = [float(err[i * 32:(i + 1) * 32].max()) for i in range(8)]
+    print("max error per 32-query block:", ["%.2e" % e for e in per_block], flush=True)
+    assert max(per_block) <= 2e-2
+    for fp8 in (False, True):   # the same map through the fp8 instantiation and with the running-max softmax
+        w = torch.full((D,), 4.0)
+        out = _call(q, k, v, block_mask=bm, fp8_qk=fp8, q_norm_weight=w.cuda(), k_norm_weight=_ones())
+        r = O.reference_layer(q, k, v, tile_map=tm, fp8_qk=fp8, q_norm_weight=w, k_norm_weight=torch.ones(D), bf16_operands=not fp8)
+        e = (out.double() - r)[0, :, 0]
+        cos = [float(torch.nn.functional.cosine_similarity(out.double()[0, i * 32:(i + 1) * 32, 0].flatten(),
+                                                           r[0, i * 32:(i + 1) * 32, 0].flatten(), dim=0)) for i in range(8)]
+        assert min(cos) >= (0.995 if fp8 else 0.9999), cos
+
+
 def test_block_sparse_full_map_equals_dense():
     import pika_h3_flex_amd as pk
 
