@@ -11,14 +11,18 @@ What follows the reference, and what is this build's own choice:
   (geometry.py:40-42) and the float64 position grid (packing.py:128).
 * The positions themselves come from a builder in the reference's un-vendored diffusers pin, which is
   not available: video rows carry their (frame, patch row, patch column), audio rows their latent index
-  on the t axis only, text rows position 0, a keyframe row the grid of the frame it anchors.  These are
-  switches of this build, not verified against the reference's module.
+  on the t axis only, text rows position 0, a keyframe row the grid of the frame it anchors, a reference
+  clip its own grid from a caller-chosen first frame.  These are switches of this build, not verified
+  against the reference's module.
+* :func:`prepare_document` and :func:`x0_from_velocity` restate what the reference's wrapper does around the
+  model call (src/pika_h3/core/wrapper.py:96-205 and :249-262): condition rows noised once and pinned, rows
+  concatenated per modality with the condition rows first, per-row timesteps, ``x0 = x_t + sigma * v``.
 """
 from __future__ import annotations
 
 from collections import OrderedDict
 from dataclasses import dataclass
-from typing import Sequence, Tuple
+from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -29,6 +33,7 @@ VIDEO_LATENT_CHANNELS = 24     #                                       -- geomet
 AUDIO_CHANNELS = 2             #                                       -- geometry.py:31
 AUDIO_LATENT_CHANNELS = 32     #                                       -- geometry.py:30
 VIDEO_TAG, TEXT_TAG, AUDIO_TAG = 0, 1, 2  #                            -- geometry.py:40-42
+KEYFRAME_NOISE_AUG = 0.999     # clean-time at which visual anchors are pinned -- wrapper.py:22-25
 
 
 # ---------------------------------------------------------------------------------------------
@@ -103,12 +108,13 @@ class PackedTokenCount:
 
 
 def packed_token_count(*, num_text_tokens: int, num_latent_frames: int, latent_height: int, latent_width: int,
-                       num_audio_latents: int, num_keyframes: int = 0, reference_audio_rows: int = 0) -> PackedTokenCount:
+                       num_audio_latents: int, num_keyframes: int = 0, reference_video_rows: int = 0,
+                       reference_audio_rows: int = 0) -> PackedTokenCount:
     """Segment sizes of one document (src/pika_h3/core/geometry.py:95-117)."""
     per_frame = (latent_height // PATCH_SIZE[1]) * (latent_width // PATCH_SIZE[2])
     return PackedTokenCount(
         text=int(num_text_tokens),
-        condition_video=int(num_keyframes) * per_frame,
+        condition_video=int(num_keyframes) * per_frame + int(reference_video_rows),
         condition_audio=int(reference_audio_rows),
         audio=int(num_audio_latents) * AUDIO_CHANNELS,
         video=int(num_latent_frames) * per_frame,
@@ -145,37 +151,109 @@ class PackedLayout:
         return torch.ones_like(m) if text else m
 
 
-def build_layout(*, num_text_tokens: int, num_latent_frames: int, latent_height: int, latent_width: int,
-                 num_audio_latents: int, keyframe_frames: Sequence[int] = (), reference_audio_rows: int = 0) -> PackedLayout:
-    """Positions, tags and index sets of one document: text, keyframe (condition video) rows, condition audio
-    rows, audio, video -- the packed order of the reference (geometry.py:83-92, wrapper.py:171-172).
+@dataclass(frozen=True)
+class ReferenceSpec:
+    """What the layout needs to know of one reference clip: its kind ("image", "video" or "audio") and whether
+    a video carries a soundtrack (src/pika_h3/core/packing.py:58-63)."""
 
-    ``keyframe_frames`` lists, per keyframe anchor, the latent frame it pins; its rows get that frame's grid.
+    kind: str
+    has_audio: bool = False
+
+
+_ANCHOR_FRAME = {"first": 0, "last": -1}
+
+
+def build_layout(text_token_tags: Optional[torch.Tensor] = None, *, num_text_tokens: Optional[int] = None,
+                 num_latent_frames: int, latent_height: int, latent_width: int, num_audio_latents: int,
+                 keyframe_anchors: Sequence[str] = (), keyframe_frames: Sequence[int] = (),
+                 references: Optional[Sequence[ReferenceSpec]] = None,
+                 reference_video_shapes: Optional[Sequence[Tuple[int, int, int]]] = None,
+                 reference_audio_rows=None, reference_first_frame: Optional[Sequence[float]] = None) -> PackedLayout:
+    """Positions, tags and index sets of one document: text, condition video rows (keyframes, or the visual
+    references), condition audio rows, audio, video -- the packed order of the reference (geometry.py:83-92,
+    wrapper.py:171-172).  Argument list after src/pika_h3/core/packing.py:154-166.
+
+    ``text_token_tags`` are the tags of the prompt rows (text 1, rows of a vision block 0, wrapper.py:18); they
+    are passed through to ``token_tags``; ``num_text_tokens`` alone means all-text.  ``keyframe_anchors`` pins
+    "first" / "last" to latent frame 0 / F-1 (``keyframe_frames`` names the frames directly); a keyframe's rows
+    get that frame's grid.  Reference ``k`` of kind image/video has latent shape ``reference_video_shapes[j]`` =
+    (frames, height, width) and gets its own grid starting at frame ``reference_first_frame[j]`` (0 by default);
+    audio references (kind audio, or a video with a soundtrack) bring ``reference_audio_rows[j]`` rows each,
+    numbered from 0 on the t axis.  ``reference_audio_rows`` may also be one integer (no ``references`` needed).
     """
-    if min(num_text_tokens, num_audio_latents, reference_audio_rows) < 0:
+    if text_token_tags is not None:
+        text_tags = text_token_tags.detach().to("cpu", torch.int64).reshape(-1)
+        if num_text_tokens is not None and int(num_text_tokens) != text_tags.numel():
+            raise ValueError("num_text_tokens disagrees with text_token_tags")
+    else:
+        if num_text_tokens is None or int(num_text_tokens) < 0:
+            raise ValueError("row counts must be >= 0")
+        text_tags = torch.full((int(num_text_tokens),), TEXT_TAG, dtype=torch.int64)
+    if num_audio_latents < 0:
         raise ValueError("row counts must be >= 0")
     hp, wp = latent_height // PATCH_SIZE[1], latent_width // PATCH_SIZE[2]
     if latent_height % PATCH_SIZE[1] or latent_width % PATCH_SIZE[2] or min(hp, wp, num_latent_frames) < 1:
         raise ValueError("latent geometry must be positive and a multiple of the patch size")
+    frames: List[int] = []
+    for a in keyframe_anchors:
+        if a not in _ANCHOR_FRAME:
+            raise ValueError(f"keyframe anchor must be 'first' or 'last', got {a!r}")
+        frames.append(_ANCHOR_FRAME[a] % num_latent_frames)
     for f in keyframe_frames:
         if not 0 <= int(f) < num_latent_frames:
             raise ValueError(f"keyframe frame {f} outside 0..{num_latent_frames - 1}")
-    counts = packed_token_count(num_text_tokens=num_text_tokens, num_latent_frames=num_latent_frames,
+        frames.append(int(f))
+    # references: visual ones take the next entry of reference_video_shapes, audible ones of reference_audio_rows
+    ref_grids: List[torch.Tensor] = []
+    if isinstance(reference_audio_rows, int):
+        audio_rows = [int(reference_audio_rows)]
+        if references:
+            raise ValueError("with references, reference_audio_rows lists one count per audible reference")
+    else:
+        audio_rows = [int(n) for n in (reference_audio_rows or [])]
+    if min(audio_rows, default=0) < 0:
+        raise ValueError("row counts must be >= 0")
+    if references:
+        if frames:
+            raise ValueError("a document carries keyframes or references, not both (wrapper.py:116-163)")
+        shapes = list(reference_video_shapes or [])
+        n_visual = sum(r.kind in ("image", "video") for r in references)
+        n_audible = sum(r.kind == "audio" or (r.kind == "video" and r.has_audio) for r in references)
+        if any(r.kind not in ("image", "video", "audio") for r in references):
+            raise ValueError("reference kind must be image, video or audio")
+        if n_visual != len(shapes) or n_audible != len(audio_rows):
+            raise ValueError(f"{n_visual} visual / {n_audible} audible references need as many shapes / row counts, "
+                             f"got {len(shapes)} / {len(audio_rows)}")
+        first = list(reference_first_frame) if reference_first_frame is not None else [0.0] * len(shapes)
+        if len(first) != len(shapes):
+            raise ValueError("reference_first_frame needs one entry per visual reference")
+        for (rf, rh, rw), f0 in zip(shapes, first):
+            if rh % PATCH_SIZE[1] or rw % PATCH_SIZE[2] or min(rf, rh, rw) < 1:
+                raise ValueError("reference latent geometry must be positive and a multiple of the patch size")
+            g = video_position_ids(int(rf), rh // PATCH_SIZE[1], rw // PATCH_SIZE[2])
+            g[:, 0] += float(f0)
+            ref_grids.append(g)
+    elif reference_video_shapes:
+        raise ValueError("reference_video_shapes without references")
+    n_ref_video = sum(int(g.shape[0]) for g in ref_grids)
+    counts = packed_token_count(num_text_tokens=text_tags.numel(), num_latent_frames=num_latent_frames,
                                 latent_height=latent_height, latent_width=latent_width,
-                                num_audio_latents=num_audio_latents, num_keyframes=len(keyframe_frames),
-                                reference_audio_rows=reference_audio_rows)
+                                num_audio_latents=num_audio_latents, num_keyframes=len(frames),
+                                reference_video_rows=n_ref_video, reference_audio_rows=sum(audio_rows))
     frame_grid = video_position_ids(1, hp, wp)
     pos, tags = [], []
     pos.append(torch.zeros((counts.text, 3), dtype=torch.float64))
-    tags.append(torch.full((counts.text,), TEXT_TAG, dtype=torch.int64))
-    for f in keyframe_frames:
+    tags.append(text_tags)
+    for f in frames:
         g = frame_grid.clone()
         g[:, 0] = float(f)
         pos.append(g)
-        tags.append(torch.full((g.shape[0],), VIDEO_TAG, dtype=torch.int64))
-    cond_a = torch.zeros((counts.condition_audio, 3), dtype=torch.float64)
-    cond_a[:, 0] = torch.arange(counts.condition_audio, dtype=torch.float64)
-    pos.append(cond_a)
+    pos.extend(ref_grids)
+    tags.append(torch.full((counts.condition_video,), VIDEO_TAG, dtype=torch.int64))
+    for n in audio_rows:
+        cond_a = torch.zeros((n, 3), dtype=torch.float64)
+        cond_a[:, 0] = torch.arange(n, dtype=torch.float64)
+        pos.append(cond_a)
     tags.append(torch.full((counts.condition_audio,), AUDIO_TAG, dtype=torch.int64))
     pos.append(audio_position_ids(num_audio_latents, AUDIO_CHANNELS))
     tags.append(torch.full((counts.audio,), AUDIO_TAG, dtype=torch.int64))
@@ -199,7 +277,7 @@ def build_layout(*, num_text_tokens: int, num_latent_frames: int, latent_height:
 
 
 def row_timesteps(layout: PackedLayout, *, video_t: float, audio_t: float, condition_video_t: float,
-                  condition_audio_t: float = 1.0, text_t: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
+                  condition_audio_t: float = 1.0, text_t: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """(unique timesteps ``[K]`` float32 ascending, per-row index ``[S]`` int32 into them): the ``timestep`` /
     ``timestep_indices`` pair of the model call (src/pika_h3/core/wrapper.py:182-190,196-197), by which every
     block gathers its AdaLN parameters per row (patches/0001-h3-adaln-fp32.patch:39-40).
@@ -207,18 +285,18 @@ def row_timesteps(layout: PackedLayout, *, video_t: float, audio_t: float, condi
     Argument list as in src/pika_h3/core/packing.py:212-231: target video rows sit at ``video_t``, target audio
     rows at ``audio_t``, condition rows at their pinned times (the wrapper passes ``max(video_t, noise_aug)``
     and 1.0, clean-time convention).  The rule itself lives in the reference's un-vendored diffusers pin
-    (``build_row_timesteps``); what that file alone fixes is a switch here: text rows take ``text_t`` (clean by
-    default) and the unique values are listed in ascending order.
+    (``build_row_timesteps``).  Text rows inherit the video time, as the wrapper states (wrapper.py:22-25);
+    ``text_t`` overrides that.  The order of the unique values is this build's choice: ascending.
     """
     S = layout.sequence_length
-    t = torch.full((S,), float(text_t), dtype=torch.float64)
+    t = torch.full((S,), float(video_t if text_t is None else text_t), dtype=torch.float64)
     n_cv, n_ca = layout.num_condition_video_rows, layout.num_condition_audio_rows
     vi, ai = layout.video_indices.cpu(), layout.audio_indices.cpu()
     t[vi[:n_cv]] = float(condition_video_t)
     t[vi[n_cv:]] = float(video_t)
     t[ai[:n_ca]] = float(condition_audio_t)
     t[ai[n_ca:]] = float(audio_t)
-    if layout.num_text_tokens == 0 and vi.numel() + ai.numel() != S:
+    if layout.num_text_tokens + vi.numel() + ai.numel() != S:
         raise ValueError("layout rows are not covered by its index sets")
     unique, index = torch.unique(t, sorted=True, return_inverse=True)
     return unique.to(torch.float32), index.to(torch.int32)
@@ -237,7 +315,14 @@ class LayoutCache:
         self.hits = self.misses = 0
 
     def get(self, **geometry) -> PackedLayout:
-        key = tuple(sorted((k, tuple(v) if isinstance(v, (list, tuple)) else v) for k, v in geometry.items()))
+        def hashable(v):
+            if isinstance(v, torch.Tensor):
+                return tuple(v.reshape(-1).tolist())
+            if isinstance(v, (list, tuple)):
+                return tuple(hashable(x) for x in v)
+            return v
+
+        key = tuple(sorted((k, hashable(v)) for k, v in geometry.items()))
         item = self._items.get(key)
         if item is not None:
             self._items.move_to_end(key)
@@ -249,3 +334,124 @@ class LayoutCache:
         if len(self._items) > self.capacity:
             self._items.popitem(last=False)
         return item
+
+
+# ---------------------------------------------------------------------------------------------
+# one document around the model call
+def _scalar_sigma(sigma, name: str) -> float:
+    """One noise level per modality (src/pika_h3/core/wrapper.py:60-69): a float, or a tensor ``[1]`` / ``[1, n]``
+    whose entries are all equal."""
+    if not isinstance(sigma, torch.Tensor):
+        return float(sigma)
+    s = sigma.detach().float().reshape(sigma.shape[0] if sigma.dim() else 1, -1)
+    if s.shape[0] != 1:
+        raise ValueError(f"{name}: one document per forward (batch size 1), got {s.shape[0]}")
+    if s.numel() > 1 and not bool(torch.all(s == s[0, 0])):
+        raise ValueError(f"{name}: one timestep per modality; per-frame values must be equal")
+    return float(s[0, 0])
+
+
+def noise_condition_rows(entry: Dict[str, Any], key: str, *, noise_aug: float = KEYFRAME_NOISE_AUG,
+                         generator: Optional[torch.Generator] = None) -> torch.Tensor:
+    """Rows of a visual anchor at clean-time ``noise_aug``: ``x = t*x0 + (1 - t)*eps``.  The noise is drawn once
+    and the rows are kept on the entry (``"_noised_rows"``), so every denoising step of a request sees the same
+    anchors (src/pika_h3/core/wrapper.py:80-94)."""
+    latents = entry[key]
+    cached = entry.get("_noised_rows")
+    if cached is not None and cached.device == latents.device:
+        return cached
+    noise = torch.randn(latents.shape, device=latents.device, dtype=torch.float32, generator=generator)
+    rows = video_latents_to_rows(noise_aug * latents.float() + (1.0 - noise_aug) * noise)
+    entry["_noised_rows"] = rows
+    return rows
+
+
+def prepare_document(video: torch.Tensor, audio: torch.Tensor, conditional_dict: Dict[str, Any], sigma_v, sigma_a, *,
+                     keyframe_noise_aug: float = KEYFRAME_NOISE_AUG, layouts: Optional[LayoutCache] = None,
+                     generator: Optional[torch.Generator] = None):
+    """The keyword tensors of one model call, as the reference's wrapper assembles them
+    (src/pika_h3/core/wrapper.py:96-205): ``(model_inputs, target_video_rows, target_audio_rows, n_cond_video,
+    n_cond_audio)``.
+
+    ``video`` ``[1, F, 24, H, W]`` and ``audio`` ``[1, T, 64]`` are the noisy target latents; ``conditional_dict``
+    carries ``prompt_embeds``, ``text_token_tags`` and optionally ``keyframes`` (``{"anchor", "latents"}``) or
+    ``references`` (``{"kind", "video_latents", "audio_latents"}``), see src/pika_h3/core/wrapper.py:16-24.
+    Visual anchors are noised once to ``keyframe_noise_aug`` and pinned at ``max(t_video, keyframe_noise_aug)``,
+    audio references stay clean at 1.0, text rows follow the video time.  ``model_inputs`` holds
+    ``hidden_states``, ``audio_hidden_states``, ``encoder_hidden_states``, ``timestep``, ``timestep_indices``,
+    ``token_tags``, ``position_ids``, ``video_indices``, ``audio_indices``, ``text_indices`` (wrapper.py:192-204);
+    ``position_ids`` and ``timestep_indices`` are what the attention processor and the AdaLN / gate gathers of
+    this package take.
+    """
+    if video.dim() != 5 or audio.dim() != 3 or video.shape[0] != 1 or audio.shape[0] != 1:
+        raise ValueError("one packed document per call: video [1, F, C, H, W] and audio [1, T, 64]")
+    device = video.device
+    _, F, C, H, W = video.shape
+    T = audio.shape[1]
+    if C != VIDEO_LATENT_CHANNELS:
+        raise ValueError(f"video latents must have {VIDEO_LATENT_CHANNELS} channels, got {C}")
+    sv, sa = _scalar_sigma(sigma_v, "sigma_v"), _scalar_sigma(sigma_a, "sigma_a")
+    t_video, t_audio = 1.0 - sv, 1.0 - sa
+    prompt = conditional_dict["prompt_embeds"]
+    if prompt.dim() == 2:
+        prompt = prompt.unsqueeze(0)
+    text_tags = conditional_dict["text_token_tags"].reshape(-1)
+    keyframes = list(conditional_dict.get("keyframes") or [])
+    references = list(conditional_dict.get("references") or [])
+    layout = conditional_dict.get("_packed_layout")
+    build = (layouts.get if layouts is not None else build_layout)
+
+    cond_video, cond_audio = [], []
+    geometry = dict(text_token_tags=text_tags, num_latent_frames=F, latent_height=H, latent_width=W, num_audio_latents=T)
+    if references:
+        specs, shapes, audio_rows = [], [], []
+        for ref in references:
+            kind = str(ref["kind"])
+            has_audio = ref.get("audio_latents") is not None
+            specs.append(ReferenceSpec(kind=kind, has_audio=has_audio if kind == "video" else kind == "audio"))
+            if kind in ("image", "video"):
+                lat = ref["video_latents"]
+                shapes.append((int(lat.shape[1]), int(lat.shape[3]), int(lat.shape[4])))
+                cond_video.append(noise_condition_rows(ref, "video_latents", noise_aug=keyframe_noise_aug,
+                                                       generator=generator).to(device))
+            if kind == "audio" or (kind == "video" and has_audio):
+                rows = audio_latents_to_rows(ref["audio_latents"].to(device).float())
+                audio_rows.append(int(rows.shape[1]))
+                cond_audio.append(rows)
+        geometry.update(references=tuple(specs), reference_video_shapes=tuple(shapes), reference_audio_rows=tuple(audio_rows))
+    else:
+        for k in keyframes:
+            if tuple(k["latents"].shape[1:]) != (1, C, H, W):
+                raise ValueError(f"keyframe latents must be [1, 1, {C}, {H}, {W}], got {tuple(k['latents'].shape)}")
+            cond_video.append(noise_condition_rows(k, "latents", noise_aug=keyframe_noise_aug, generator=generator).to(device))
+        geometry.update(keyframe_anchors=tuple(str(k["anchor"]) for k in keyframes))
+    if layout is None:
+        layout = build(**geometry)
+    layout_dev = conditional_dict.get("_packed_layout_device")
+    if layout_dev is None or layout_dev.position_ids.device != device:
+        layout_dev = layout.to(device)
+
+    target_video = video_latents_to_rows(video.float())
+    target_audio = audio_latents_to_rows(audio.float())
+    video_rows = torch.cat(cond_video + [target_video], dim=1) if cond_video else target_video
+    audio_rows_all = torch.cat(cond_audio + [target_audio], dim=1) if cond_audio else target_audio
+    if video_rows.shape[1] != layout.video_indices.numel() or audio_rows_all.shape[1] != layout.audio_indices.numel():
+        raise ValueError(f"packed rows disagree with the layout: video {video_rows.shape[1]} vs {layout.video_indices.numel()}, "
+                         f"audio {audio_rows_all.shape[1]} vs {layout.audio_indices.numel()}")
+    unique_t, t_index = row_timesteps(layout, video_t=t_video, audio_t=t_audio,
+                                      condition_video_t=max(t_video, keyframe_noise_aug), condition_audio_t=1.0)
+    model_inputs = dict(
+        hidden_states=video_rows, audio_hidden_states=audio_rows_all, encoder_hidden_states=prompt.to(device),
+        timestep=unique_t.to(device), timestep_indices=t_index.to(device), token_tags=layout_dev.token_tags,
+        position_ids=layout_dev.position_ids, video_indices=layout_dev.video_indices,
+        audio_indices=layout_dev.audio_indices, text_indices=layout_dev.text_indices, return_dict=False)
+    return model_inputs, target_video, target_audio, layout.num_condition_video_rows, layout.num_condition_audio_rows
+
+
+def x0_from_velocity(target_rows: torch.Tensor, velocity_rows: torch.Tensor, sigma, n_condition_rows: int = 0) -> torch.Tensor:
+    """``x0 = x_t + sigma * v`` in fp32 on the target rows only: the model returns a velocity for every row of the
+    modality, condition rows first, and those are dropped (src/pika_h3/core/wrapper.py:249-262)."""
+    v = velocity_rows[:, n_condition_rows:]
+    if v.shape != target_rows.shape:
+        raise ValueError(f"velocity rows {tuple(v.shape)} do not match the target rows {tuple(target_rows.shape)}")
+    return target_rows.float() + _scalar_sigma(sigma, "sigma") * v.float()

@@ -118,11 +118,116 @@ def test_row_timesteps_per_segment():
     assert uniq.dtype == torch.float32 and idx.dtype == torch.int32 and idx.shape == (53,)
     assert uniq.tolist() == [0.25, 0.5, 0.75, 1.0]
     per_row = uniq[idx.long()].tolist()
-    # text (clean), keyframe rows (pinned), condition audio (clean), audio, video
-    assert per_row == [1.0] * 5 + [0.75] * 12 + [1.0] * 4 + [0.5] * 14 + [0.25] * 18
+    # text (follows the video time, src/pika_h3/core/wrapper.py:22-25), keyframe rows (pinned), condition audio
+    # (clean), audio, video
+    assert per_row == [0.25] * 5 + [0.75] * 12 + [1.0] * 4 + [0.5] * 14 + [0.25] * 18
     # equal times share one entry: video and audio at the same time, keyframes no noisier than the video
     uniq, idx = P.row_timesteps(lay, video_t=0.5, audio_t=0.5, condition_video_t=0.5)
-    assert uniq.tolist() == [0.5, 1.0] and idx.tolist() == [1] * 5 + [0] * 12 + [1] * 4 + [0] * 32
+    assert uniq.tolist() == [0.5, 1.0] and idx.tolist() == [0] * 5 + [0] * 12 + [1] * 4 + [0] * 32
     # the text switch
-    uniq, idx = P.row_timesteps(lay, video_t=0.5, audio_t=0.5, condition_video_t=0.5, condition_audio_t=0.5, text_t=0.5)
+    uniq, idx = P.row_timesteps(lay, video_t=0.5, audio_t=0.5, condition_video_t=0.5, condition_audio_t=0.5, text_t=1.0)
+    assert uniq.tolist() == [0.5, 1.0] and idx.tolist() == [1] * 5 + [0] * 48
+    uniq, idx = P.row_timesteps(lay, video_t=0.5, audio_t=0.5, condition_video_t=0.5, condition_audio_t=0.5)
     assert uniq.tolist() == [0.5] and int(idx.abs().sum()) == 0
+
+
+def test_layout_text_tags_anchors_and_references():
+    """Argument list of src/pika_h3/core/packing.py:154-166: prompt tags pass through, "first"/"last" anchors,
+    references with their own latent shapes and audio rows; segment sizes as src/pika_h3/core/geometry.py:95-117."""
+    tags = torch.tensor([1, 1, 0, 0, 0, 1])          # a vision block inside the prompt (wrapper.py:18)
+    lay = P.build_layout(tags, num_latent_frames=3, latent_height=4, latent_width=6, num_audio_latents=2,
+                         keyframe_anchors=("first", "last"))
+    assert lay.token_tags[:6].tolist() == tags.tolist() and lay.num_text_tokens == 6
+    assert lay.counts == P.packed_token_count(num_text_tokens=6, num_latent_frames=3, latent_height=4, latent_width=6,
+                                              num_audio_latents=2, num_keyframes=2)
+    kf = lay.position_ids[lay.video_indices[:12]]
+    assert kf[:6, 0].tolist() == [0.0] * 6 and kf[6:, 0].tolist() == [2.0] * 6
+    assert torch.equal(kf[:6, 1:], lay.position_ids[lay.video_indices[12:18], 1:])   # the grid of the pinned frame
+    with pytest.raises(ValueError):
+        P.build_layout(tags, num_latent_frames=3, latent_height=4, latent_width=6, num_audio_latents=2, keyframe_anchors=("middle",))
+
+    refs = (P.ReferenceSpec("image"), P.ReferenceSpec("video", has_audio=True), P.ReferenceSpec("audio"))
+    lay = P.build_layout(num_text_tokens=2, num_latent_frames=3, latent_height=4, latent_width=6, num_audio_latents=2,
+                         references=refs, reference_video_shapes=((1, 8, 4), (2, 4, 4)), reference_audio_rows=(6, 4),
+                         reference_first_frame=(0.0, 10.0))
+    assert lay.counts == P.packed_token_count(num_text_tokens=2, num_latent_frames=3, latent_height=4, latent_width=6,
+                                              num_audio_latents=2, reference_video_rows=8 + 8, reference_audio_rows=10)
+    assert lay.sequence_length == 2 + 16 + 10 + 4 + 18
+    cv = lay.position_ids[lay.video_indices[:16]]
+    assert cv[:8, 0].tolist() == [0.0] * 8 and cv[7].tolist() == [0.0, 3.0, 1.0]          # 4 x 2 patches of the image
+    assert cv[8:, 0].tolist() == [10.0] * 4 + [11.0] * 4
+    ca = lay.position_ids[lay.audio_indices[:10]]
+    assert ca[:, 0].tolist() == list(range(6)) + list(range(4)) and float(ca[:, 1:].abs().sum()) == 0
+    assert set(lay.token_tags[lay.video_indices].tolist()) == {P.VIDEO_TAG}
+    assert set(lay.token_tags[lay.audio_indices].tolist()) == {P.AUDIO_TAG}
+    every = torch.cat([lay.text_indices, lay.video_indices, lay.audio_indices]).sort().values
+    assert torch.equal(every, torch.arange(lay.sequence_length))
+    for bad in (dict(reference_video_shapes=((1, 8, 4),)), dict(reference_audio_rows=(6,)),
+                dict(reference_first_frame=(0.0,)), dict(keyframe_anchors=("first",))):
+        kw = dict(references=refs, reference_video_shapes=((1, 8, 4), (2, 4, 4)), reference_audio_rows=(6, 4))
+        kw.update(bad)
+        with pytest.raises(ValueError):
+            P.build_layout(num_text_tokens=2, num_latent_frames=3, latent_height=4, latent_width=6, num_audio_latents=2, **kw)
+
+
+def _document(F=3, H=4, W=6, T=5, L=4):
+    g = torch.Generator().manual_seed(3)
+    video = torch.randn(1, F, 24, H, W, generator=g)
+    audio = torch.randn(1, T, 64, generator=g)
+    cond = {"prompt_embeds": torch.randn(L, 16, generator=g), "text_token_tags": torch.ones(1, L, dtype=torch.long)}
+    return video, audio, cond, g
+
+
+def test_prepare_document_keyframes():
+    """Mirror of src/pika_h3/core/wrapper.py:96-205 for the first/last-frame task."""
+    video, audio, cond, g = _document()
+    cond["keyframes"] = [{"anchor": "first", "latents": torch.randn(1, 1, 24, 4, 6, generator=g)},
+                         {"anchor": "last", "latents": torch.randn(1, 1, 24, 4, 6, generator=g)}]
+    cache = P.LayoutCache()
+    mi, tv, ta, ncv, nca = P.prepare_document(video, audio, cond, torch.tensor([0.75]), torch.tensor([[0.5, 0.5]]),
+                                              layouts=cache, generator=torch.Generator().manual_seed(1))
+    assert (ncv, nca) == (12, 0) and tv.shape == (1, 18, 96) and ta.shape == (1, 10, 32)
+    assert set(mi) == {"hidden_states", "audio_hidden_states", "encoder_hidden_states", "timestep", "timestep_indices",
+                       "token_tags", "position_ids", "video_indices", "audio_indices", "text_indices", "return_dict"}
+    assert mi["hidden_states"].shape == (1, 30, 96) and torch.equal(mi["hidden_states"][:, 12:], tv)
+    assert mi["encoder_hidden_states"].shape == (1, 4, 16) and mi["position_ids"].shape == (4 + 12 + 10 + 18, 3)
+    # the anchors: t*x0 + (1-t)*eps at t = 0.999, so within 0.1 % noise of the clean rows, and not equal to them
+    clean = P.video_latents_to_rows(cond["keyframes"][0]["latents"])
+    got = mi["hidden_states"][:, :6]
+    assert not torch.equal(got, clean) and float((got - 0.999 * clean).abs().max()) < 0.001 * 6
+    # per-row times: text and video at 1 - 0.75, audio at 0.5, anchors pinned at max(0.25, 0.999)
+    per_row = mi["timestep"][mi["timestep_indices"].long()]
+    want = torch.tensor([0.25] * 4 + [0.999] * 12 + [0.5] * 10 + [0.25] * 18)
+    assert torch.allclose(per_row, want) and mi["timestep"].tolist() == sorted(mi["timestep"].tolist())
+    # the second denoising step reuses the layout and the same noised anchors
+    mi2, *_ = P.prepare_document(video, audio, cond, 0.5, 0.5, layouts=cache)
+    assert cache.hits == 1 and torch.equal(mi2["hidden_states"][:, :12], mi["hidden_states"][:, :12])
+    assert mi2["timestep"].tolist() == pytest.approx([0.5, 0.999])
+    # x0 = x_t + sigma*v on the target rows only
+    v = torch.randn(1, 30, 96)
+    x0 = P.x0_from_velocity(tv, v, torch.tensor([0.75]), ncv)
+    assert torch.allclose(x0, tv + 0.75 * v[:, 12:])
+    assert torch.equal(P.video_rows_to_latents(tv, 3, 4, 6), video)
+    with pytest.raises(ValueError):
+        P.x0_from_velocity(tv, v, 0.75, 0)
+    with pytest.raises(ValueError):
+        P.prepare_document(video, audio, cond, torch.tensor([[0.1, 0.2]]), 0.5)            # per-frame sigmas differ
+    with pytest.raises(ValueError):
+        P.prepare_document(video.expand(2, -1, -1, -1, -1), audio, cond, 0.5, 0.5)         # one document per call
+
+
+def test_prepare_document_references():
+    video, audio, cond, g = _document()
+    cond["references"] = [{"kind": "image", "video_latents": torch.randn(1, 1, 24, 8, 4, generator=g)},
+                          {"kind": "video", "video_latents": torch.randn(1, 2, 24, 4, 4, generator=g),
+                           "audio_latents": torch.randn(1, 3, 64, generator=g)},
+                          {"kind": "audio", "audio_latents": torch.randn(1, 2, 64, generator=g)}]
+    mi, tv, ta, ncv, nca = P.prepare_document(video, audio, cond, 0.5, 0.25)
+    assert (ncv, nca) == (8 + 8, 6 + 4)
+    assert mi["hidden_states"].shape[1] == ncv + 18 and mi["audio_hidden_states"].shape[1] == nca + 10
+    # audio references are packed clean and sit at time 1.0
+    assert torch.equal(mi["audio_hidden_states"][:, :6], P.audio_latents_to_rows(cond["references"][1]["audio_latents"]))
+    per_row = mi["timestep"][mi["timestep_indices"].long()]
+    ai = mi["audio_indices"]
+    assert per_row[ai[:nca]].tolist() == [1.0] * nca and per_row[ai[nca:]].tolist() == [0.75] * 10
+    assert per_row[mi["video_indices"][:ncv]].tolist() == pytest.approx([0.999] * ncv)
