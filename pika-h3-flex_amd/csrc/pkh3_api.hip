@@ -439,7 +439,7 @@ int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream)
       if (!lin[t]->lora_a_img) continue;
       GemmTarget& tg = g.tg[g.n_targets++];
       tg = GemmTarget{};
-      tg.epi = kEpiKImg; tg.n = PKH3_LORA_RANK; tg.n_tiles = 1;
+      tg.epi = kEpiAImg; tg.n = PKH3_LORA_RANK; tg.n_tiles = 1;
       tg.w_img = (const char*)lin[t]->lora_a_img; tg.w_blk_stride = w_blk;
       tg.out_scale = lin[t]->lora_scale;
       tg.out = (char*)p->lora_workspace + t * b_blk; tg.out_head_stride = 0;
@@ -511,7 +511,7 @@ int pkh3_out_proj(const pkh3_out_args* p, void* stream) {
     g.n_targets = 1; g.n_tiles = 1;
     GemmTarget& tg = g.tg[0];
     tg = GemmTarget{};
-    tg.epi = kEpiKImg; tg.n = PKH3_LORA_RANK; tg.n_tiles = 1;
+    tg.epi = kEpiAImg; tg.n = PKH3_LORA_RANK; tg.n_tiles = 1;
     tg.w_img = (const char*)p->proj.lora_a_img; tg.w_blk_stride = w_blk; tg.out_scale = p->proj.lora_scale;
     tg.out = (char*)p->lora_workspace; tg.out_blk_stride = 2 * b_blk; tg.out_sub_stride = (int)b_blk;
     if ((e = launch_gemm(g, st)) != hipSuccess) return hip_fail(e, "lora down-projection");

@@ -2,24 +2,24 @@
 //
 // Work split.  A workgroup is 12 waves (dense; three per SIMD) or 8 waves (block-sparse; two per SIMD);
 // each wave owns 32 queries of one (batch, head) and keeps for them, in VGPRs, the Q operand images, the
-// running row max / row sum and the fp32 output accumulator O^T (128 x 32).  All waves share every 64-key
+// running row max / row sum and the fp32 output accumulator O^T (128 x 32, sixteen 16x16 blocks).  All waves share every 64-key
 // K/V tile, which is copied HBM/L2 -> LDS with direct-to-LDS loads into a 3-slot ring, two tiles ahead of
 // the math.  Several waves per SIMD is what overlaps the softmax VALU work of one wave with the MFMAs of
 // another; the whole per-wave state stays in VGPRs (<= 168 dense, <= 256 sparse) so no accumulator ever
 // moves between register files.  Q is read in place: RMSNorm, rotation and fp8 quantisation of the Q rows
 // happen in registers while the first K/V tiles are in flight.
 //
-// Math per tile, all on the 32x32 MFMA shapes (see pkh3_common.h for the operand images):
-//   S^T = K' Q'^T      A = K image (LDS), B = Q image (VGPR)      -> lane l holds query l%32, 16 keys / block
-//                      (bf16: 16 x 32x32x16, Q' carries softmax_scale * log2(e) so S^T is in the log2 domain;
-//                      fp8: 4 x 32x32x64 on e4m3 images, S^T rescaled by the per-64-row-block dequantisation
-//                      scales in the softmax multiply)
+// Math per tile, all on the 16x16 MFMA shapes (see pkh3_common.h for the operand images and why these shapes):
+//   S^T = K' Q'^T      A = K image (LDS), B = Q image (VGPR)      -> lane l holds queries l%16 and 16 + l%16, 4 keys
+//                      per 16-key block (bf16: 32 x 16x16x32, Q' carries softmax_scale * log2(e) so S^T is in the
+//                      log2 domain; fp8: 8 x 16x16x128 on e4m3 images, S^T rescaled by the per-64-row-block
+//                      dequantisation scales in the softmax multiply)
 //   softmax            bounded-logit path (the usual one): |q_i| * max_j |k_j| bounds every logit of the wave's
 //                      queries; when that bound is small, exp2(logit) needs no maximum at all.  Otherwise the
-//                      online form: row max in-lane over the keys + one exchange with lane l^32, raised only
-//                      when exceeded by 2^8 so the O^T rescale is rare.  Row sum kept per half-wave, merged once
-//                      at the end.
-//   O^T += V^T P^T     A = V image (LDS), B = P packed to bf16 straight from the S^T registers
+//                      online form: row max in-lane over the keys + two row swaps across the four lane groups,
+//                      raised only when exceeded by 2^8 so the O^T rescale is rare.  Row sum kept per lane group,
+//                      merged once at the end.
+//   O^T += V^T P^T     A = V image (LDS), B = P packed to bf16 straight from the S^T registers (32 x 16x16x32)
 // The transposed formulation keeps every per-query quantity (max, sum, rescale factor) a per-lane
 // scalar: no cross-lane traffic in the rescale, none between the two GEMMs.  O leaves through LDS, turned
 // around into whole 256-byte rows.
@@ -48,14 +48,18 @@ constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when ex
 constexpr float kStaticMaxLimit = 48.0f;  // rows whose |logit| bound is below this skip the running max (terms 2^-48 .. 2^48)
 
 #define PKH3_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-// Each tile loop ends on an 8-pass MFMA into the O^T accumulators.  The compiler was seen to place the register
+// Each tile loop ends on an MFMA into the O^T accumulators.  The compiler was seen to place the register
 // copies that merge the two loop variants (v_mov_b64 reading the accumulator's last registers) four scalar
 // instructions after that MFMA, before its result is written back; the block-sparse kernel then returned a stale
 // O^T block.  32 idle issue cycles after every loop let the last MFMA retire whatever follows.  The accumulators
 // are operands of the statement, so every read or copy of them the compiler emits after the loop is ordered
 // after the idle cycles.
-#define PKH3_MFMA_DRAIN(W) \
-  asm volatile("s_nop 15\n\ts_nop 15" : "+v"((W).o[0]), "+v"((W).o[1]), "+v"((W).o[2]), "+v"((W).o[3])::"memory")
+#define PKH3_MFMA_DRAIN(W)                                                                                               \
+  asm volatile("s_nop 15\n\ts_nop 15"                                                                                    \
+               : "+v"((W).o[0][0]), "+v"((W).o[0][1]), "+v"((W).o[1][0]), "+v"((W).o[1][1]), "+v"((W).o[2][0]),          \
+                 "+v"((W).o[2][1]), "+v"((W).o[3][0]), "+v"((W).o[3][1]), "+v"((W).o[4][0]), "+v"((W).o[4][1]),          \
+                 "+v"((W).o[5][0]), "+v"((W).o[5][1]), "+v"((W).o[6][0]), "+v"((W).o[6][1]), "+v"((W).o[7][0]),          \
+                 "+v"((W).o[7][1])::"memory")
 constexpr int kSgMfma = 0x008, kSgDsRead = 0x100;
 
 __device__ __forceinline__ void lds_dma16(const char* g, unsigned lane_off, char* l) {
@@ -79,44 +83,51 @@ __device__ __forceinline__ T uniform_load(const T* p, int i) {
   return ((const __attribute__((address_space(4))) T*)p)[i];
 }
 
-__device__ __forceinline__ float max_across_halves(float x) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+// maximum over the four lanes l % 16 == const (one per 16-lane group): two row swaps, no LDS crossbar
+__device__ __forceinline__ float max_across_groups(float x) {
+  const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(r16[0]), __uint_as_float(r16[1]));
+  const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r32[0]), __uint_as_float(r32[1]));
 }
 
+// Per-wave state.  Lane (c = l % 16, g = l / 16) works for the two queries 16*qb + c, qb = 0, 1, of the wave's 32.
 template <bool FP8>
 struct WaveState {
-  bf16x8 qf[FP8 ? 1 : 8];  // bf16 Q images, one per 16-wide k-step
-  i32x4 q8[FP8 ? 4 : 1];   // fp8 Q images, 16 B chunks (two per 64-wide k-step)
-  f32x16 s[2];             // S^T of the tile: two blocks of 32 keys
-  f32x16 o[4];             // O^T accumulators: four blocks of 32 head-dim rows
-  bf16x8 vf[8];            // V images of the first 32 keys, fetched while QK^T finishes
-  float m, l;              // running row max (scaled, log2 domain), per-half-wave row sum
+  bf16x8 qf[FP8 ? 1 : 2][FP8 ? 1 : 4];  // bf16 Q images (qb, ks): Q'[16*qb + c][32*ks + 8*g + j]
+  i32x8 q8[FP8 ? 2 : 1];                // fp8 Q images (qb): bytes 8*ks + j = element 32*ks + 8*g + j
+  f32x4 s[4][2];                        // S^T of the tile (kb, qb): keys 16*kb + 4*g + i
+  f32x4 o[8][2];                        // O^T accumulators (db, qb): head-dim rows 16*db + 4*g + i
+  bf16x8 vf[8];                         // V images of the first 32 keys, fetched while QK^T finishes
+  float m[2], l[2];                     // per query block: running row max (scaled, log2 domain), this lane group's row sum
 };
 
-// S^T = K' Q'^T for the 64 keys of one tile.  LDS reads run 8 images ahead of the MFMAs that consume
-// them; the tail of the MFMA chain covers the first V image reads.
+#define PKH3_MFMA16(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, B, C, 0, 0, 0)
+// format codes 0/0 = e4m3 x e4m3; scale operands 0 select the unscaled form of the instruction
+#define PKH3_MFMA16_F8(A, B, C) __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C, 0, 0, 0, 0, 0, 0)
+
+// S^T = K' Q'^T for the 64 keys of one tile: image i of the K tile is (half, ks, kb2) = (i >> 3, (i >> 1) & 3, i & 1)
+// and feeds the two query blocks, so four accumulators rotate inside each half.  LDS reads run 8 images ahead of
+// the MFMAs that consume them; the tail of the MFMA chain covers the first V image reads.
 // LEAN (three waves per SIMD, 168 VGPRs): the reads run only 4 images ahead and V is left to the P.V loop.
 template <bool FP8, bool LEAN>
 __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane) {
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) w.s[kb][i] = 0.f;
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   if constexpr (!FP8 && LEAN) {
     bf16x8 kf[16];
 #pragma unroll
     for (int i = 0; i < 4; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int kb = i >> 3, ks = i & 7;
-      w.s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], w.qf[ks], w.s[kb], 0, 0, 0);
+      const int ks = (i >> 1) & 3, kb = 2 * (i >> 3) + (i & 1);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.s[kb][qb] = PKH3_MFMA16(kf[i], w.qf[qb][ks], ks == 0 ? zero : w.s[kb][qb]);
       if (i + 4 < 16) kf[i + 4] = *(const bf16x8*)(kbuf + ((i + 4) * 64 + lane) * 16);
     }
     PKH3_SGB(kSgDsRead, 4);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      PKH3_SGB(kSgMfma, 1);
+      PKH3_SGB(kSgMfma, 2);
       if (i + 4 < 16) PKH3_SGB(kSgDsRead, 1);
     }
   } else if constexpr (!FP8) {
@@ -125,8 +136,9 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
     for (int i = 0; i < 8; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int kb = i >> 3, ks = i & 7;
-      w.s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], w.qf[ks], w.s[kb], 0, 0, 0);
+      const int ks = (i >> 1) & 3, kb = 2 * (i >> 3) + (i & 1);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.s[kb][qb] = PKH3_MFMA16(kf[i], w.qf[qb][ks], ks == 0 ? zero : w.s[kb][qb]);
       if (i < 8)
         kf[i + 8] = *(const bf16x8*)(kbuf + ((i + 8) * 64 + lane) * 16);
       else
@@ -135,7 +147,7 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
     PKH3_SGB(kSgDsRead, 8);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      PKH3_SGB(kSgMfma, 1);
+      PKH3_SGB(kSgMfma, 2);
       PKH3_SGB(kSgDsRead, 1);
     }
   } else {
@@ -143,31 +155,22 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
 #pragma unroll
     for (int i = 0; i < 8; ++i) kc[i] = *(const i32x4*)(kbuf + (i * 64 + lane) * 16);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int kb = i >> 1, ks = i & 1;
-      const i32x4 a0 = kc[kb * 4 + 2 * ks], a1 = kc[kb * 4 + 2 * ks + 1];
-      const i32x4 b0 = w.q8[2 * ks], b1 = w.q8[2 * ks + 1];
+    for (int kb = 0; kb < 4; ++kb) {
+      const i32x4 a0 = kc[2 * kb], a1 = kc[2 * kb + 1];
       const i32x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-      const i32x8 b = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
-      // format codes 0/0 = e4m3 x e4m3; scale operands 0 select the unscaled form of the instruction
-      w.s[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, w.s[kb], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.s[kb][qb] = PKH3_MFMA16_F8(a, w.q8[qb], zero);
       // the MFMA chain covers the first V image reads: 8 images, or 4 where registers are short (LEAN)
       if constexpr (LEAN) {
-        w.vf[i] = *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
+        w.vf[kb] = *(const bf16x8*)(vbuf + (kb * 64 + lane) * 16);
       } else {
-        w.vf[2 * i] = *(const bf16x8*)(vbuf + ((2 * i) * 64 + lane) * 16);
-        w.vf[2 * i + 1] = *(const bf16x8*)(vbuf + ((2 * i + 1) * 64 + lane) * 16);
+        w.vf[2 * kb] = *(const bf16x8*)(vbuf + ((2 * kb) * 64 + lane) * 16);
+        w.vf[2 * kb + 1] = *(const bf16x8*)(vbuf + ((2 * kb + 1) * 64 + lane) * 16);
       }
     }
   }
 }
 
-// Softmax numerators of w.s, then O^T += V^T P^T.  `c` = softmax scale * log2(e) (times the fp8
-// dequantisation scales of this tile); `lim` = keys of this tile that exist (only read when < 64).
-// STATIC: w.m holds a per-query upper bound of every logit (|q_i| * max_j |k_j| * c), small enough that
-// exp2(logit - bound) cannot underflow; the running max, its exchange across the half-waves and the
-// O^T rescale are then not needed at all, and the numerators of the first 32 keys do not wait for the
-// second half of S^T.
 // exp2 of one logit.  bf16 path: Q' already carries softmax_scale * log2(e), so S^T is in the log2 domain and
 // `c` is unused; fp8 path: `c` carries that factor times the dequantisation scales.  STATIC: the logits are
 // bounded in magnitude (see kStaticMaxLimit), so no maximum is subtracted at all.
@@ -177,89 +180,114 @@ __device__ __forceinline__ float softmax_numerator(float s, float c, float m) {
   else return __builtin_amdgcn_exp2f(STATIC ? s : s - m);
 }
 
-template <bool FP8, bool STATIC, bool LEAN, bool MASKED>
-__device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* vbuf, float c, int lim, int lane) {
-  const int hh = lane >> 5;
-  if constexpr (MASKED) {
+// Softmax numerators of NKB key blocks of w.s (a whole tile: 4, a 32-key half: 2) into the P^T operands of
+// the P.V MFMAs: operand (half, qb) takes, for lane group g, the keys v_image_key(g, j) of its half, i.e. registers
+// 0..3 of key block 2*half and of key block 2*half + 1 -- P never leaves its lane.  Also the running max / rescale
+// of the online path and the row sums.  `lim` = keys of these blocks that exist (only read when MASKED).
+// STATIC: w.m is not used: every logit is bounded (|q_i| * max_j |k_j| * c), small enough that exp2(logit) is a
+// normal number; the running max, its exchange across the lane groups and the O^T rescale are then not needed at
+// all, and the numerators of the first 32 keys do not wait for the second half of S^T.
+template <bool FP8, bool STATIC, bool MASKED, int NKB>
+__device__ __forceinline__ void softmax_blocks(WaveState<FP8>& w, bf16x8 (&pf)[NKB / 2][2], float c, int lim, int lane) {
+  const int g = lane >> 4;
+  if (MASKED) {
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = kb * 32 + 8 * (i / 4) + 4 * hh + (i % 4);
-        if (key >= lim) w.s[kb][i] = -INFINITY;
-      }
+      for (int i = 0; i < 4; ++i)
+        if (16 * kb + 4 * g + i >= lim) {
+          w.s[kb][0][i] = -INFINITY;
+          w.s[kb][1][i] = -INFINITY;
+        }
   }
-  float m_new = w.m, alpha = 1.0f;
+  float m_new[2] = {w.m[0], w.m[1]}, alpha[2] = {1.0f, 1.0f};
   if constexpr (!STATIC) {
-    float mx = fmaxf(w.s[0][0], w.s[1][0]);
 #pragma unroll
-    for (int i = 1; i < 16; ++i) mx = fmaxf(fmaxf(mx, w.s[0][i]), w.s[1][i]);
-    mx = max_across_halves(mx) * (FP8 ? c : 1.0f);
-    m_new = (mx > w.m + kRescaleSlack) ? mx : w.m;
-    alpha = __builtin_amdgcn_exp2f(w.m - m_new);
-    w.m = m_new;
-    if (__any(alpha != 1.0f)) {
+    for (int qb = 0; qb < 2; ++qb) {
+      float mx = w.s[0][qb][0];
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) w.o[db][i] *= alpha;
+        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, w.s[kb][qb][i]);
+      mx = max_across_groups(mx) * (FP8 ? c : 1.0f);
+      m_new[qb] = (mx > w.m[qb] + kRescaleSlack) ? mx : w.m[qb];
+      alpha[qb] = __builtin_amdgcn_exp2f(w.m[qb] - m_new[qb]);
+      w.m[qb] = m_new[qb];
+    }
+    if (__any(alpha[0] != 1.0f || alpha[1] != 1.0f)) {
+#pragma unroll
+      for (int db = 0; db < 8; ++db)
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) w.o[db][qb][i] *= alpha[qb];
     }
   }
-  bf16x8 pf[2][2];
-  float rsum = 0.f;
   const bf16x2 one2 = {(__bf16)1.0f, (__bf16)1.0f};
+  float rsum[2] = {0.f, 0.f};
 #pragma unroll
-  for (int kb = 0; kb < 2; ++kb)
+  for (int half = 0; half < NKB / 2; ++half)
 #pragma unroll
-    for (int b2 = 0; b2 < 2; ++b2) {
+    for (int qb = 0; qb < 2; ++qb) {
       bf16x8 pk;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) pk[j] = (__bf16)softmax_numerator<FP8, STATIC>(w.s[kb][8 * b2 + j], c, m_new);
+      for (int j = 0; j < 8; ++j)
+        pk[j] = (__bf16)softmax_numerator<FP8, STATIC>(w.s[2 * half + (j >> 2)][qb][j & 3], c, m_new[qb]);
       // row sum over the bf16-rounded values, the same numbers the P.V MFMA consumes
 #pragma unroll
       for (int j = 0; j < 8; j += 2) {
         const bf16x2 pr = {pk[j], pk[j + 1]};
-        rsum = __builtin_amdgcn_fdot2_f32_bf16(pr, one2, rsum, false);
+        rsum[qb] = __builtin_amdgcn_fdot2_f32_bf16(pr, one2, rsum[qb], false);
       }
-      pf[kb][b2] = pk;
+      pf[half][qb] = pk;
     }
-  w.l = STATIC ? w.l + rsum : w.l * alpha + rsum;
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) w.l[qb] = STATIC ? w.l[qb] + rsum[qb] : w.l[qb] * alpha[qb] + rsum[qb];
+}
+
+// Softmax of w.s, then O^T += V^T P^T for one tile: V image i is (half, db) = (i >> 3, i & 7) and feeds the two
+// query blocks, sixteen accumulators in rotation.  `c` = softmax scale * log2(e) (times the fp8 dequantisation
+// scales of this tile); `lim` = keys of this tile that exist (only read when MASKED).
+template <bool FP8, bool STATIC, bool LEAN, bool MASKED>
+__device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* vbuf, float c, int lim, int lane) {
+  bf16x8 pf[2][2];
+  softmax_blocks<FP8, STATIC, MASKED, 4>(w, pf, c, lim, lane);
   if constexpr (LEAN) {
     bf16x8 vg[16];
 #pragma unroll
     for (int i = 0; i < 4; ++i) vg[i] = FP8 ? w.vf[i] : *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int kb = i >> 3, b2 = (i >> 2) & 1, db = i & 3;
-      w.o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vg[i], pf[kb][b2], w.o[db], 0, 0, 0);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.o[i & 7][qb] = PKH3_MFMA16(vg[i], pf[i >> 3][qb], w.o[i & 7][qb]);
       if (i + 4 < 16) vg[i + 4] = *(const bf16x8*)(vbuf + ((i + 4) * 64 + lane) * 16);
     }
   } else {
     bf16x8 vg[8];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int kb = i >> 3, b2 = (i >> 2) & 1, db = i & 3;
-      w.o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(i < 8 ? w.vf[i] : vg[i - 8], pf[kb][b2], w.o[db], 0, 0, 0);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.o[i & 7][qb] = PKH3_MFMA16(i < 8 ? w.vf[i] : vg[i - 8], pf[i >> 3][qb], w.o[i & 7][qb]);
       if (i < 8) vg[i] = *(const bf16x8*)(vbuf + ((i + 8) * 64 + lane) * 16);
     }
   }
 }
 
-// ---- 32-key half tiles, used by the second phase of the block-sparse kernel -----------------------------
-// S^T (32 keys x 32 queries) into w.s[0]; kbuf/vbuf point at this half's K images (8 bf16 / 4 fp8 chunks)
+// ---- 32-key half tiles: the short-key and split forms of the dense kernel, phase 2 of the block-sparse one ----
+// S^T (32 keys x 32 queries) into w.s[0..1]; kbuf/vbuf point at this half's K images (8 bf16 / 4 fp8 chunks)
 // and V images (8).
 // LEAN (three waves per SIMD): the K reads run 4 images ahead and only the fp8 path prefetches V (4 images).
 template <bool FP8, bool LEAN = false>
 __device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane) {
-#pragma unroll
-  for (int i = 0; i < 16; ++i) w.s[0][i] = 0.f;
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   if constexpr (!FP8 && LEAN) {
     bf16x8 kf[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      w.s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], w.qf[i], w.s[0], 0, 0, 0);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.s[i & 1][qb] = PKH3_MFMA16(kf[i], w.qf[qb][i >> 1], i < 2 ? zero : w.s[i & 1][qb]);
       if (i + 4 < 8) kf[i + 4] = *(const bf16x8*)(kbuf + ((i + 4) * 64 + lane) * 16);
     }
   } else if constexpr (!FP8) {
@@ -268,7 +296,8 @@ __device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, con
     for (int i = 0; i < 8; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      w.s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], w.qf[i], w.s[0], 0, 0, 0);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.s[i & 1][qb] = PKH3_MFMA16(kf[i], w.qf[qb][i >> 1], i < 2 ? zero : w.s[i & 1][qb]);
       w.vf[i] = *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
     }
   } else {
@@ -276,79 +305,44 @@ __device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, con
 #pragma unroll
     for (int i = 0; i < 4; ++i) kc[i] = *(const i32x4*)(kbuf + (i * 64 + lane) * 16);
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const i32x4 a0 = kc[2 * ks], a1 = kc[2 * ks + 1];
-      const i32x4 b0 = w.q8[2 * ks], b1 = w.q8[2 * ks + 1];
+    for (int kb = 0; kb < 2; ++kb) {
+      const i32x4 a0 = kc[2 * kb], a1 = kc[2 * kb + 1];
       const i32x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-      const i32x8 b = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
-      w.s[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, w.s[0], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.s[kb][qb] = PKH3_MFMA16_F8(a, w.q8[qb], zero);
 #pragma unroll
       for (int i = 0; i < (LEAN ? 2 : 4); ++i) {
-        const int v = (LEAN ? 2 : 4) * ks + i;
+        const int v = (LEAN ? 2 : 4) * kb + i;
         w.vf[v] = *(const bf16x8*)(vbuf + (v * 64 + lane) * 16);
       }
     }
   }
 }
 
-// Softmax numerators of w.s[0] and O^T += V^T P^T for one half tile (V images already in w.vf).
+// Softmax numerators of w.s[0..1] and O^T += V^T P^T for one half tile (V images already in w.vf).
 // `lim` = keys of this half that exist (<= 0: none; only read when < 32).
 // LEAN: the V images (beyond the 4 the fp8 path prefetched) are read here, 4 ahead of their MFMAs, from vbuf.
 // FULL: the caller guarantees lim == 32, no masking code at all.
 template <bool FP8, bool STATIC, bool LEAN = false, bool FULL = false>
 __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int lim, int lane, const char* vbuf = nullptr) {
-  const int hh = lane >> 5;
-  if (!FULL && lim < 32) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = 8 * (i / 4) + 4 * hh + (i % 4);
-      if (key >= lim) w.s[0][i] = -INFINITY;
-    }
-  }
-  float m_new = w.m, alpha = 1.0f;
-  if constexpr (!STATIC) {
-    float mx = w.s[0][0];
-#pragma unroll
-    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, w.s[0][i]);
-    mx = max_across_halves(mx) * (FP8 ? c : 1.0f);
-    m_new = (mx > w.m + kRescaleSlack) ? mx : w.m;
-    alpha = __builtin_amdgcn_exp2f(w.m - m_new);
-    w.m = m_new;
-    if (__any(alpha != 1.0f)) {
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) w.o[db][i] *= alpha;
-    }
-  }
-  bf16x8 pf[2];
-  float rsum = 0.f;
-  const bf16x2 one2 = {(__bf16)1.0f, (__bf16)1.0f};
-#pragma unroll
-  for (int b2 = 0; b2 < 2; ++b2) {
-    bf16x8 pk;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) pk[j] = (__bf16)softmax_numerator<FP8, STATIC>(w.s[0][8 * b2 + j], c, m_new);
-#pragma unroll
-    for (int j = 0; j < 8; j += 2) {
-      const bf16x2 pr = {pk[j], pk[j + 1]};
-      rsum = __builtin_amdgcn_fdot2_f32_bf16(pr, one2, rsum, false);
-    }
-    pf[b2] = pk;
-  }
-  w.l = STATIC ? w.l + rsum : w.l * alpha + rsum;
+  bf16x8 pf[1][2];
+  if (!FULL && lim < 32) softmax_blocks<FP8, STATIC, true, 2>(w, pf, c, lim, lane);
+  else softmax_blocks<FP8, STATIC, false, 2>(w, pf, c, lim, lane);
   if constexpr (LEAN) {
     bf16x8 vg[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) vg[i] = FP8 ? w.vf[i] : *(const bf16x8*)(vbuf + (i * 64 + lane) * 16);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      w.o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vg[i], pf[i >> 2], w.o[i & 3], 0, 0, 0);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.o[i][qb] = PKH3_MFMA16(vg[i], pf[0][qb], w.o[i][qb]);
       if (i + 4 < 8) vg[i + 4] = *(const bf16x8*)(vbuf + ((i + 4) * 64 + lane) * 16);
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) w.o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w.vf[i], pf[i >> 2], w.o[i & 3], 0, 0, 0);
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) w.o[i][qb] = PKH3_MFMA16(w.vf[i], pf[0][qb], w.o[i][qb]);
   }
 }
 
@@ -382,7 +376,7 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   constexpr int kPhase2Bytes = SPARSE ? kStages2 * kSparseRows * kHalfBytes : 0;
   constexpr int kRingBytes = HALFMODE ? GROUPS * kRing * kHalfBytes
                              : (kPhase2Bytes > kRingT * kTileBytes ? kPhase2Bytes : kRingT * kTileBytes);
-  constexpr int kMergeBytes = 64 * 64 * 4 + 2 * 64 * 4;  // SPLIT: one wave's O^T, row sums and row maxima in fp32
+  constexpr int kMergeBytes = 64 * 64 * 4 + 4 * 64 * 4;  // SPLIT: one wave's O^T, row sums and row maxima in fp32
   constexpr int kAfterBytes = SPLIT ? kShortWaves * kMergeBytes : WAVES * kStageBytes;  // LDS use after the loops
   constexpr int kLdsBytes = kRingBytes > kAfterBytes ? kRingBytes : kAfterBytes;
   __shared__ __attribute__((aligned(1024))) char lds_raw[kLdsBytes];
@@ -467,7 +461,7 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     if (kAhead > 1 && nt > 1) dma(entry(1), 1);
   }
   // Q load, fused with QK-RMSNorm, rotation and (fp8) quantisation: lane (l%32, hh) reads the 64 elements
-  // d = 16*ks + 8*hh + j of query row q32*32 + l%32 -- the ones it carries in the MFMA B images -- so the
+  // d = 16*ks + 8*hh + j of query row q32*32 + l%32 (whole 8-element pieces of the MFMA B images), so the
   // operand images are formed in registers and Q' never exists in memory.
   float qscale = 1.0f;
   float qn2 = 0.f;  // squared norm of the (rounded / dequantised) Q' row: this lane's half, then the full row
@@ -478,15 +472,34 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     load_row(x, (const __bf16*)p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh + (int64_t)(valid ? qrow : 0) * p.q_ss, valid, hh);
     const RowTransform tf{p.q_norm_w, p.q_eps, p.q_rope_mode, p.q_cos, p.q_sin};
     norm_rope_row(x, tf, qrow, valid, hh);
+    // The row math above works two lanes per row (the layout of norm_rope_row); the MFMA operand wants four lanes per
+    // row: lane (c, g) carries, for query block qb, the pieces p8 = 4*ks + g of row 16*qb + c.  Those sit in lane
+    // 32*(g%2) + 16*qb + c as its pieces ks8 = 2*ks + g/2: one lane permutation per piece, done once per workgroup.
+    const int g4 = lane >> 4, src_base = 32 * (g4 & 1) + (lane & 15);
+    const bool odd = (g4 >> 1) != 0;
     if constexpr (!FP8) {
+      bf16x8 qold[8];
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           // softmax_scale * log2(e) rides in Q', so S^T comes out of the MFMAs in the log2 domain
           const __bf16 r = (__bf16)(x[ks * 8 + j] * p.c);
-          w.qf[ks][j] = r;
+          qold[ks][j] = r;
           qn2 = fmaf((float)r, (float)r, qn2);
+        }
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          const i32x4 e = __builtin_bit_cast(i32x4, qold[2 * ks]), o = __builtin_bit_cast(i32x4, qold[2 * ks + 1]);
+          i32x4 t;
+#pragma unroll
+          for (int wd = 0; wd < 4; ++wd) {
+            const int ve = __shfl(e[wd], src_base + 16 * qb, 64), vo = __shfl(o[wd], src_base + 16 * qb, 64);
+            t[wd] = odd ? vo : ve;
+          }
+          w.qf[qb][ks] = __builtin_bit_cast(bf16x8, t);
         }
     } else {
       // one absmax scale per 64-query block = this wave and its neighbour (wave ^ 1)
@@ -500,26 +513,39 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
       amax = fmaxf(amax, q_amax[wave ^ 1]);
       qscale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
       const float inv = 1.0f / qscale;
+      i32x4 qold[4];
 #pragma unroll
       for (int c4 = 0; c4 < 4; ++c4) {
-        w.q8[c4] = quant_fp8_chunk(x, c4, inv);
+        qold[c4] = quant_fp8_chunk(x, c4, inv);
 #pragma unroll
         for (int wd = 0; wd < 4; ++wd) {
-          const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w.q8[c4][wd], false);
-          const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(w.q8[c4][wd], true);
+          const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(qold[c4][wd], false);
+          const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(qold[c4][wd], true);
           qn2 += lo[0] * lo[0] + lo[1] * lo[1] + hi[0] * hi[0] + hi[1] * hi[1];
         }
       }
       qn2 *= qscale * qscale;
+      // chunk c4 of the two-lane layout holds the pieces ks8 = 2*c4 (words 0, 1) and 2*c4 + 1 (words 2, 3)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+          for (int wd = 0; wd < 2; ++wd) {
+            const int ve = __shfl(qold[ks][wd], src_base + 16 * qb, 64), vo = __shfl(qold[ks][2 + wd], src_base + 16 * qb, 64);
+            w.q8[qb][2 * ks + wd] = odd ? vo : ve;
+          }
     }
     qn2 += xhalf(qn2);
   }
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < 8; ++db)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) w.o[db][i] = 0.f;
-  w.m = -INFINITY;
-  w.l = 0.f;
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w.o[db][qb][i] = 0.f;
+  w.m[0] = w.m[1] = -INFINITY;
+  w.l[0] = w.l[1] = 0.f;
   const float c = p.c * qscale;
   const float* kscale = FP8 ? p.kscale + (int64_t)bh * p.nKt : nullptr;
   const int tail = sk & (kTileKeys - 1);  // keys in the last tile when it is partial
@@ -594,34 +620,35 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
       for (int src = 1; src < GROUPS; ++src) {
         if (group == src) {
 #pragma unroll
-          for (int db = 0; db < 4; ++db)
+          for (int db = 0; db < 8; ++db)
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-              const f32x4 v4 = {w.o[db][4 * g4], w.o[db][4 * g4 + 1], w.o[db][4 * g4 + 2], w.o[db][4 * g4 + 3]};
-              *(f32x4*)(mbuf + ((db * 4 + g4) * 64 + lane) * 4) = v4;
-            }
-          mbuf[64 * 64 + lane] = w.l;
-          mbuf[64 * 64 + 64 + lane] = w.m;
+            for (int qb = 0; qb < 2; ++qb) *(f32x4*)(mbuf + ((db * 2 + qb) * 64 + lane) * 4) = w.o[db][qb];
+#pragma unroll
+          for (int qb = 0; qb < 2; ++qb) {
+            mbuf[64 * 64 + qb * 64 + lane] = w.l[qb];
+            mbuf[64 * 64 + 128 + qb * 64 + lane] = w.m[qb];
+          }
         }
         __syncthreads();
         if (group == 0) {
-          const float l2 = mbuf[64 * 64 + lane], m2 = mbuf[64 * 64 + 64 + lane];
-          float a1 = 1.0f, a2 = 1.0f;
-          if (!static_max) {
-            const float mn = fmaxf(w.m, m2);
-            a1 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w.m - mn);
-            a2 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m2 - mn);
-            w.m = mn;
-          }
-          w.l = w.l * a1 + l2 * a2;
 #pragma unroll
-          for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-              const f32x4 v4 = *(const f32x4*)(mbuf + ((db * 4 + g4) * 64 + lane) * 4);
-#pragma unroll
-              for (int rr = 0; rr < 4; ++rr) w.o[db][4 * g4 + rr] = w.o[db][4 * g4 + rr] * a1 + v4[rr] * a2;
+          for (int qb = 0; qb < 2; ++qb) {
+            const float l2 = mbuf[64 * 64 + qb * 64 + lane], m2 = mbuf[64 * 64 + 128 + qb * 64 + lane];
+            float a1 = 1.0f, a2 = 1.0f;
+            if (!static_max) {
+              const float mn = fmaxf(w.m[qb], m2);
+              a1 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w.m[qb] - mn);
+              a2 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m2 - mn);
+              w.m[qb] = mn;
             }
+            w.l[qb] = w.l[qb] * a1 + l2 * a2;
+#pragma unroll
+            for (int db = 0; db < 8; ++db) {
+              const f32x4 v4 = *(const f32x4*)(mbuf + ((db * 2 + qb) * 64 + lane) * 4);
+#pragma unroll
+              for (int rr = 0; rr < 4; ++rr) w.o[db][qb][rr] = w.o[db][qb][rr] * a1 + v4[rr] * a2;
+            }
+          }
         }
         __syncthreads();
       }
@@ -696,27 +723,32 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
 #undef PKH3_HALF_LOOP
   }
 
-  // Epilogue: O = O^T / l in bf16.  A lane holds 4 consecutive d of one query per register group, which would
-  // make 8-byte stores scattered over 32 rows; instead each wave turns its 32 x 128 block around in its own
-  // 8 KiB of LDS (16-byte chunks XOR-swizzled by the row so both directions are conflict-free) and stores
-  // whole 256-byte rows, 16 bytes per lane.
+  // Epilogue: O = O^T / l in bf16.  A lane holds 4 consecutive d of a query per accumulator, which would make 8-byte
+  // stores scattered over 16 rows; instead each wave turns its 32 x 128 block around in its own 8 KiB of LDS
+  // (16-byte chunks XOR-swizzled by the row so both directions are conflict-free) and stores whole 256-byte rows,
+  // 16 bytes per lane.
   __bf16* ob = (__bf16*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
-  const float lt = w.l + xhalf(w.l);
-  const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+  float inv[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const float lt = wave_sum_groups(w.l[qb]);
+    inv[qb] = lt > 0.f ? 1.0f / lt : 0.f;
+  }
   __syncthreads();  // every wave is done reading K/V tiles (SPLIT: and merge buffers): the LDS becomes staging space
   if (SPLIT && group != 0) return;  // the merged result lives in group 0
   char* stage = lds_raw + wq * kStageBytes;
   {
-    const int qr = lane & 31;
+    const int c16 = lane & 15, g = lane >> 4;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int db = 0; db < 8; ++db) {
         bf16x4 wv;
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr) wv[rr] = (__bf16)(w.o[db][4 * g + rr] * inv);
-        const int chunk = (4 * db + g) ^ (qr & 15);
-        *(bf16x4*)(stage + qr * 256 + chunk * 16 + 8 * hh) = wv;
+        for (int rr = 0; rr < 4; ++rr) wv[rr] = (__bf16)(w.o[db][qb][rr] * inv[qb]);
+        // elements d = 16*db + 4*g .. +3 of row 16*qb + c16: 16-byte chunk 2*db + g/2, its half g%2
+        const int chunk = (2 * db + (g >> 1)) ^ c16;
+        *(bf16x4*)(stage + (16 * qb + c16) * 256 + chunk * 16 + 8 * (g & 1)) = wv;
       }
   }
   // same wave wrote and reads: the LDS counter orders the two, no barrier

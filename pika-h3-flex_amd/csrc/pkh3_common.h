@@ -1,25 +1,32 @@
-// Shared device-side definitions for the gfx950 attention kernels: vector types, the fragment
-// ("frag") layouts the prologue writes and the attention kernels consume, and small wave helpers.
+// Shared device-side definitions for the gfx950 attention kernels: vector types, the operand-image
+// layouts the prologue (or the projection GEMM's epilogue) writes and the attention kernel consumes,
+// and small wave helpers.
 //
-// Fragment layouts.  All matrix work uses the CDNA4 32x32 MFMA shapes.  For those, lane l of a
-// wave supplies row/column (l % 32) of an operand and a contiguous run of the contraction index
-// selected by its half hh = l / 32; the 32x32 fp32 result puts column (l % 32) in lane l and rows
-// 8*(i/4) + 4*hh + (i%4) in its 16 registers i.  The prologue stores Q, K and V in HBM already cut
-// into 1 KiB operand images (64 lanes x 16 B), so the attention kernel moves them HBM -> LDS ->
-// VGPR as straight 16-byte copies with no shuffles and no LDS bank conflicts.
+// Operand images.  The attention kernel runs on the CDNA4 16x16 MFMA shapes (16x16x32 bf16, 16x16x128 fp8):
+// at the same peak rate they move a quarter of the accumulator registers per instruction of the 32x32 shapes,
+// and the part sustains about 10 % more of them per second on real data.  For those shapes lane l of a wave
+// supplies row/column c = l % 16 of an operand and the 8 consecutive contraction elements selected by its group
+// g = l / 16; the 16x16 fp32 result puts column c in lane l and rows 4*g + i in its 4 registers i.  K and V are
+// stored in HBM already cut into 1 KiB images (64 lanes x 16 B) in exactly that order, so the attention kernel
+// moves them HBM -> LDS -> VGPR as straight 16-byte copies with no shuffles and no LDS bank conflicts.
 //
-//   K tile (64 keys, bf16): image (kb, ks), kb in 0..1, ks in 0..7, at byte ((kb*8+ks)*64 + l)*16
-//       holds K'[32*kb + l%32][16*ks + 8*hh + j], j = 0..7            (A operand of S^T = K' Q'^T)
-//   Q block (32 queries, bf16): image ks at ((ks)*64 + l)*16 holds Q'[l%32][16*ks + 8*hh + j]
+//   K tile (64 keys, bf16, 16 KiB): image (half, ks, kb2), half in 0..1, ks in 0..3, kb2 in 0..1, at byte
+//       (((half*4 + ks)*2 + kb2)*64 + l)*16 holds K'[32*half + 16*kb2 + c][32*ks + 8*g + j], j = 0..7
+//       (A operand of S^T = K' Q'^T; the 32-key halves are contiguous for the half-tile forms of the kernel)
+//   Q block (32 queries, bf16, registers only): image (qb, ks) holds Q'[16*qb + c][32*ks + 8*g + j]
 //       (B operand of S^T)
-//   V tile (64 keys, bf16): image (kb, b2, db), b2 in 0..1, db in 0..3, at (((kb*2+b2)*4+db)*64 + l)*16
-//       holds V[32*kb + 8*(2*b2 + j/4) + 4*hh + j%4][32*db + l%32]      (A operand of O^T = V^T P^T)
-//       -- the key order is the one the S^T result registers 8*b2 .. 8*b2+7 already have, so P goes
-//       from the softmax registers into the next MFMA without leaving the lane.
-//   fp8 K tile / Q block: image (kb, ks64), 32 B per lane: byte j of lane l is element
-//       d = 16*(4*ks64 + j/8) + 8*hh + j%8 of row 32*kb + l%32 -- the same lane-to-d assignment as
-//       the bf16 images, four of them concatenated; Q and K use it alike, which is all the
+//   V tile (64 keys, bf16, 16 KiB): image (half, db), db in 0..7, at ((half*8 + db)*64 + l)*16 holds
+//       V[32*half + 16*(j/4) + 4*g + j%4][16*db + c], j = 0..7      (A operand of O^T = V^T P^T)
+//       -- the key order is the one the S^T result registers of key blocks 2*half and 2*half+1 already have,
+//       so P goes from the softmax registers into the next MFMA without leaving the lane.
+//   fp8 K tile (8 KiB): key block kb in 0..3 is 2 KiB, 32 B per lane as two 16-byte chunks c2 at
+//       ((kb*2 + c2)*64 + l)*16; byte 8*(ks%2) + j of chunk c2 = ks/2 is element d = 32*ks + 8*g + j of row
+//       16*kb + c -- the same lane-to-d assignment as the bf16 images; Q uses it alike, which is all the
 //       contraction needs.
+//
+// Rows are prepared (RMSNorm, rotation, quantisation) with two lanes per row: lane (r = l % 32, hh = l / 32)
+// holds the 64 elements d = 16*ks8 + 8*hh + j of row r, i.e. the 8-element pieces p8 = 2*ks8 + hh of the row.
+// Piece p8 of a row belongs to lane group g = p8 % 4 and k-step ks = p8 / 4 of the images above.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -134,7 +141,29 @@ __device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform
   }
 }
 
-// values 16*c .. 16*c+15 of a lane's row -> one 16-byte chunk of an fp8 e4m3 image
+__device__ __forceinline__ float wave_sum_groups(float x) {
+  // sum over the four lanes l % 16 == const (one per 16-lane group)
+  x += __shfl_xor(x, 16, 64);
+  x += __shfl_xor(x, 32, 64);
+  return x;
+}
+
+// byte offset, inside a bf16 K tile, of the 16-byte piece p8 (elements 8*p8 .. 8*p8+7) of the tile's row rt
+__device__ __forceinline__ int k_piece_offset(int rt, int p8) {
+  const int half = rt >> 5, kb2 = (rt >> 4) & 1, c = rt & 15, ks = p8 >> 2, g = p8 & 3;
+  return ((((half * 4 + ks) * 2 + kb2) * 64) + 16 * g + c) * 16;
+}
+
+// byte offset, inside an fp8 K tile, of the 16-byte chunk that holds the pieces p8 and p8 + 4 (p8 % 8 < 4) of row rt
+__device__ __forceinline__ int k8_chunk_offset(int rt, int p8) {
+  const int kb = rt >> 4, c = rt & 15, c2 = p8 >> 3, g = p8 & 3;
+  return (((kb * 2 + c2) * 64) + 16 * g + c) * 16;
+}
+
+// key (inside its 32-key half) that element j of lane group g carries in a V image / in the P operand
+__device__ __forceinline__ int v_image_key(int g, int j) { return 16 * (j >> 2) + 4 * g + (j & 3); }
+
+// values 16*c .. 16*c+15 of a lane's row -> 16 bytes of fp8 e4m3: pieces ks8 = 2c (words 0, 1) and 2c + 1 (words 2, 3)
 __device__ __forceinline__ i32x4 quant_fp8_chunk(const float (&x)[64], int c, float inv) {
   i32x4 t;
 #pragma unroll

@@ -14,7 +14,8 @@
 //   C   = x W^T  (tokens down the registers, one feature per lane)               V images
 // Weight rows are stored permuted inside each 128-feature head so that, in the C^T form, the 64 accumulator
 // values of a lane are exactly the 64 head-dim elements d = 16*ks + 8*hh + j the row transform
-// (norm_rope_row) and the K image store expect.
+// (norm_rope_row) works on: whole 8-element pieces of the row, which the epilogue stores at their places in the
+// attention kernel's K tile (a different image shape: that kernel runs on the 16x16 MFMAs, these GEMMs on 32x32).
 //
 // Work split.  Workgroup = 8 waves = 256 tokens x 256 features; wave (fh, tq) owns features fh*128..+127 (one
 // head) x tokens tq*64..+63 (one K/V tile): 8 accumulators of 32x32.  Per 32-wide k-chunk a wave reads 8 weight
@@ -161,22 +162,25 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
     if (tok0 >= p.M) break;                          // tiles past the last token: nothing to write
 
     if constexpr (EPI == kEpiVImg) {
-      // lane = feature 32*db + r of the head, registers = tokens: exactly the V image rows
+      // lane = feature 32*db + r of the head, registers = tokens 8*(i/4) + 4*hh + i%4 of a 32-token block.  The V
+      // image (half = token block, db16) wants lane (g, c) = feature 16*db16 + c with tokens 16*(j/4) + 4*g + j%4:
+      // this lane's registers 4*(2*(j/4) + a) + j%4 are that piece for g = 2*a + hh, db16 = 2*db + r/16, c = r%16.
       char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
 #pragma unroll
       for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-        for (int b2 = 0; b2 < 2; ++b2)
+        for (int a = 0; a < 2; ++a)
 #pragma unroll
           for (int db = 0; db < 4; ++db) {
             const float bv = bias ? bias[32 * db + r] : 0.f;
             bf16x8 img;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-              const int token = tok0 + 32 * t2 + 8 * (2 * b2 + j / 4) + 4 * hh + (j % 4);
-              img[j] = token < p.M ? (__bf16)(acc[2 * tp + t2][db][8 * b2 + j] + bv) : (__bf16)0.0f;
+              const int i = 4 * (2 * (j >> 2) + a) + (j & 3);
+              const int token = tok0 + 32 * t2 + 8 * (i >> 2) + 4 * hh + (i & 3);
+              img[j] = token < p.M ? (__bf16)(acc[2 * tp + t2][db][i] + bv) : (__bf16)0.0f;
             }
-            *(bf16x8*)(rec + (((t2 * 2 + b2) * 4 + db) * 64 + lane) * 16) = img;
+            *(bf16x8*)(rec + ((t2 * 8 + 2 * db + (r >> 4)) * 64 + 16 * (2 * a + hh) + (r & 15)) * 16) = img;
           }
     } else {
       // lane = token, its 64 accumulator values per token block = head-dim elements 16*ks + 8*hh + j in x[ks*8 + j]
@@ -200,7 +204,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
             }
           }
       }
-      if constexpr (EPI == kEpiKImg) {
+      if constexpr (EPI == kEpiKImg || EPI == kEpiAImg) {
         const RowTransform tf{tg.norm_w, tg.norm_eps, tg.rope_mode, tg.cos_t, tg.sin_t};
         float nmax = 0.f, amax = 0.f;
 #pragma unroll
@@ -233,7 +237,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
               bf16x8 t;
 #pragma unroll
               for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[t2][ks * 8 + j];
-              *(bf16x8*)(rec + t2 * tg.out_sub_stride + (ks * 64 + lane) * 16) = t;
+              // kEpiKImg: the attention kernel's K tile; kEpiAImg: operand images of these GEMMs ([token block][k-step])
+              if constexpr (EPI == kEpiKImg) *(bf16x8*)(rec + k_piece_offset(32 * t2 + r, 2 * ks + hh)) = t;
+              else *(bf16x8*)(rec + t2 * tg.out_sub_stride + (ks * 64 + lane) * 16) = t;
             }
         } else {
           amax = wave_max(amax);
@@ -243,8 +249,14 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
 #pragma unroll
           for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
-              *(i32x4*)(rec + t2 * tg.out_sub_stride + (c * 64 + lane) * 16) = quant_fp8_chunk(x[t2], c, inv);
+            for (int c2 = 0; c2 < 2; ++c2) {
+              const i32x4 q0 = quant_fp8_chunk(x[t2], 2 * c2, inv), q1 = quant_fp8_chunk(x[t2], 2 * c2 + 1, inv);
+#pragma unroll
+              for (int a = 0; a < 2; ++a) {
+                const i32x4 t = {q0[2 * a], q0[2 * a + 1], q1[2 * a], q1[2 * a + 1]};
+                *(i32x4*)(rec + k8_chunk_offset(32 * t2 + r, 2 * (4 * c2 + a) + hh)) = t;
+              }
+            }
         }
       } else {
         // row-major bf16 rows: y = residual + gate[row_index] * (acc*scale + bias); 16-byte pieces per lane
@@ -306,6 +318,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void gemm_kernel(GemmParams p) {
   switch (tg.epi) {
     case kEpiRows: gemm_tile<kEpiRows, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
     case kEpiKImg: gemm_tile<kEpiKImg, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
+    case kEpiAImg: gemm_tile<kEpiAImg, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
     default: gemm_tile<kEpiVImg, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
   }
 }

@@ -82,7 +82,9 @@ struct FwdParams {
 };
 
 // ---- projection GEMMs (pkh3_gemm.hip) -------------------------------------------------------------------
-enum { kEpiRows = 0, kEpiKImg = 1, kEpiVImg = 2 };       // what a target's epilogue writes
+// what a target's epilogue writes: row-major rows, the attention kernel's K tiles (norm, rotation, fp8), its V tiles,
+// or bf16 operand images of these GEMMs themselves (the LoRA down-projection feeding the second K segment)
+enum { kEpiRows = 0, kEpiKImg = 1, kEpiVImg = 2, kEpiAImg = 3 };
 enum { kNormNone = 0, kNormLayer = 1, kNormRms = 2 };    // row normalisation of the pack / modulation pass
 
 // One output of a GEMM launch: a run of `n` features (whole 128-feature heads) with its own weights and epilogue.
@@ -104,7 +106,7 @@ struct GemmTarget {
   char* out;
   int64_t out_head_stride; // image epilogues: bytes between heads
   int64_t out_blk_stride;  // image epilogues: bytes between 64-token tiles
-  int out_sub_stride;      // kEpiKImg: bytes between the two 32-token halves of a tile
+  int out_sub_stride;      // kEpiAImg: bytes between the two 32-token blocks of a 64-token pair
   int64_t out_row_stride;  // kEpiRows: elements between token rows
   int out_head_elems;      // kEpiRows: elements between heads
   // kEpiKImg

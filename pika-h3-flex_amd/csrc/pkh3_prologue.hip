@@ -54,9 +54,9 @@ hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int
 // RMSNorm + RoPE (+ fp8 quantisation) of K rows into operand images (the Q side does the same math
 // inside the attention kernel, on the rows each wave owns).
 // One wave owns one 64-row block of one (batch, head): lane (r = l%32, hh = l/32) holds, for the
-// two 32-row halves `sub`, the 64 elements d = 16*ks + 8*hh + j of row 32*sub + r -- exactly the
-// elements its lane carries in the MFMA images, so norm, rotation and the store need one
-// cross-lane exchange only (the sum of squares with lane l^32).
+// two 32-row halves `sub`, the 64 elements d = 16*ks + 8*hh + j of row 32*sub + r -- whole 16-byte
+// pieces of the operand images, so norm and rotation need one cross-lane exchange only (the sum of
+// squares with lane l^32) and the store is 16 bytes per piece at its place in the image.
 template <bool FP8>
 __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
         bf16x8 t;
 #pragma unroll
         for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[sub][ks * 8 + j];
-        *(bf16x8*)(ob + ((sub * 8 + ks) * 64 + lane) * 16) = t;
+        *(bf16x8*)(ob + k_piece_offset(32 * sub + r, 2 * ks + hh)) = t;
       }
   } else {
     float amax = 0.f;
@@ -120,8 +120,15 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        *(i32x4*)(ob + ((sub * 4 + c) * 64 + lane) * 16) = quant_fp8_chunk(x[sub], c, inv);
+      for (int c2 = 0; c2 < 2; ++c2) {
+        // this lane's pieces ks8 = 4*c2 .. 4*c2+3; pieces ks8 and ks8 + 2 share a lane group and a chunk
+        const i32x4 q0 = quant_fp8_chunk(x[sub], 2 * c2, inv), q1 = quant_fp8_chunk(x[sub], 2 * c2 + 1, inv);
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          const i32x4 t = {q0[2 * a], q0[2 * a + 1], q1[2 * a], q1[2 * a + 1]};
+          *(i32x4*)(ob + k8_chunk_offset(32 * sub + r, 2 * (4 * c2 + a) + hh)) = t;
+        }
+      }
   }
 }
 
@@ -136,37 +143,35 @@ hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st) {
 
 // ------------------------------------------------------------------------------------------------
 // V rows -> A-operand images of O^T = V^T P^T.  One wave per 64-key tile of one (batch, head).
-// Lane (r, hh) of image (kb, b2, db) needs V[key(kb,b2,hh,j)][32*db + r] for j = 0..7: eight rows at
-// one column.  Reads are 2-byte gathers (64 B contiguous per half-wave, served from L1/L2); the
+// Lane (c, g) of image (half, db) needs V[32*half + v_image_key(g, j)][16*db + c] for j = 0..7: eight rows at
+// one column.  Reads are 2-byte gathers (32 B contiguous per lane group, served from L1/L2); the
 // stores are full 1 KiB lines.
 __global__ __launch_bounds__(256) void v_prologue_kernel(VPrologueParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int t = blockIdx.y * 4 + wave;
   if (t >= p.nKt) return;
   const int h = blockIdx.x, b = blockIdx.z;  // heads fastest, as in the K prologue
-  const int r = lane & 31, hh = lane >> 5;
+  const int c = lane & 15, g = lane >> 4;
   if (t == 0 && lane == 0) p.zero_init[b * p.H + h] = 0u;
   const int rows = p.row_cnt ? p.row_cnt[b] : p.S;
   const __bf16* vb = (const __bf16*)p.v + (int64_t)b * p.sb + (int64_t)h * p.sh;
   char* ob = p.out + (int64_t)(b * p.H + h) * p.out_bh_stride + (int64_t)t * p.out_tile_stride;
 #pragma unroll
-  for (int kb = 0; kb < 2; ++kb)
+  for (int half = 0; half < 2; ++half) {
+    bf16x8 img[8];
 #pragma unroll
-    for (int b2 = 0; b2 < 2; ++b2) {
-      bf16x8 img[4];
+    for (int j = 0; j < 8; ++j) {
+      const int row = t * 64 + half * 32 + v_image_key(g, j);
+      const bool valid = row < rows;
+      int src = 0;
+      if (valid) src = p.gather_idx ? p.gather_idx[(int64_t)b * p.S + row] : row;
+      const __bf16* vr = vb + (int64_t)src * p.ss + c;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int row = t * 64 + kb * 32 + 8 * (2 * b2 + j / 4) + 4 * hh + (j % 4);
-        const bool valid = row < rows;
-        int src = 0;
-        if (valid) src = p.gather_idx ? p.gather_idx[(int64_t)b * p.S + row] : row;
-        const __bf16* vr = vb + (int64_t)src * p.ss + r;
-#pragma unroll
-        for (int db = 0; db < 4; ++db) img[db][j] = valid ? vr[32 * db] : (__bf16)0.0f;
-      }
-#pragma unroll
-      for (int db = 0; db < 4; ++db) *(bf16x8*)(ob + (((kb * 2 + b2) * 4 + db) * 64 + lane) * 16) = img[db];
+      for (int db = 0; db < 8; ++db) img[db][j] = valid ? vr[16 * db] : (__bf16)0.0f;
     }
+#pragma unroll
+    for (int db = 0; db < 8; ++db) *(bf16x8*)(ob + ((half * 8 + db) * 64 + lane) * 16) = img[db];
+  }
 }
 
 hipError_t launch_v_prologue(const VPrologueParams& p, hipStream_t st) {
