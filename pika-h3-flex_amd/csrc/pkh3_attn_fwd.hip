@@ -478,21 +478,21 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     const int g4 = lane >> 4, src_base = 32 * (g4 & 1) + (lane & 15);
     const bool odd = (g4 >> 1) != 0;
     if constexpr (!FP8) {
-      bf16x8 qold[8];
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
+      for (int ks = 0; ks < 4; ++ks) {
+        bf16x8 qold[2];  // this lane's pieces ks8 = 2*ks, 2*ks + 1 in the two-lane layout
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          // softmax_scale * log2(e) rides in Q', so S^T comes out of the MFMAs in the log2 domain
-          const __bf16 r = (__bf16)(x[ks * 8 + j] * p.c);
-          qold[ks][j] = r;
-          qn2 = fmaf((float)r, (float)r, qn2);
-        }
+        for (int a = 0; a < 2; ++a)
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb)
+          for (int j = 0; j < 8; ++j) {
+            // softmax_scale * log2(e) rides in Q', so S^T comes out of the MFMAs in the log2 domain
+            const __bf16 r = (__bf16)(x[(2 * ks + a) * 8 + j] * p.c);
+            qold[a][j] = r;
+            qn2 = fmaf((float)r, (float)r, qn2);
+          }
+        const i32x4 e = __builtin_bit_cast(i32x4, qold[0]), o = __builtin_bit_cast(i32x4, qold[1]);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          const i32x4 e = __builtin_bit_cast(i32x4, qold[2 * ks]), o = __builtin_bit_cast(i32x4, qold[2 * ks + 1]);
+        for (int qb = 0; qb < 2; ++qb) {
           i32x4 t;
 #pragma unroll
           for (int wd = 0; wd < 4; ++wd) {
@@ -501,6 +501,7 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
           }
           w.qf[qb][ks] = __builtin_bit_cast(bf16x8, t);
         }
+      }
     } else {
       // one absmax scale per 64-query block = this wave and its neighbour (wave ^ 1)
       __shared__ float q_amax[WAVES];
