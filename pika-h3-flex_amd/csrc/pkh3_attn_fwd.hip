@@ -110,25 +110,26 @@ struct WaveState {
 // and feeds the two query blocks, so four accumulators rotate inside each half.  LDS reads run 8 images ahead of
 // the MFMAs that consume them; the tail of the MFMA chain covers the first V image reads.
 // LEAN (three waves per SIMD, 168 VGPRs): the reads run only 4 images ahead and V is left to the P.V loop.
-template <bool FP8, bool LEAN>
+// AHEAD: images the LEAN reads run ahead (the copies of the loop that run once per workgroup take 2 and fit the registers)
+template <bool FP8, bool LEAN, int AHEAD = 4>
 __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane) {
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   if constexpr (!FP8 && LEAN) {
     bf16x8 kf[16];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
+    for (int i = 0; i < AHEAD; ++i) kf[i] = *(const bf16x8*)(kbuf + (i * 64 + lane) * 16);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int ks = (i >> 1) & 3, kb = 2 * (i >> 3) + (i & 1);
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb) w.s[kb][qb] = PKH3_MFMA16(kf[i], w.qf[qb][ks], ks == 0 ? zero : w.s[kb][qb]);
-      if (i + 4 < 16) kf[i + 4] = *(const bf16x8*)(kbuf + ((i + 4) * 64 + lane) * 16);
+      if (i + AHEAD < 16) kf[i + AHEAD] = *(const bf16x8*)(kbuf + ((i + AHEAD) * 64 + lane) * 16);
     }
-    PKH3_SGB(kSgDsRead, 4);
+    PKH3_SGB(kSgDsRead, AHEAD);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       PKH3_SGB(kSgMfma, 2);
-      if (i + 4 < 16) PKH3_SGB(kSgDsRead, 1);
+      if (i + AHEAD < 16) PKH3_SGB(kSgDsRead, 1);
     }
   } else if constexpr (!FP8) {
     bf16x8 kf[16];
@@ -326,7 +327,8 @@ __device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, con
 template <bool FP8, bool STATIC, bool LEAN = false, bool FULL = false>
 __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int lim, int lane, const char* vbuf = nullptr) {
   bf16x8 pf[1][2];
-  if (!FULL && lim < 32) softmax_blocks<FP8, STATIC, true, 2>(w, pf, c, lim, lane);
+  // the running-max form always takes the masking copy (two copies of it do not fit the registers of some variants)
+  if (!FULL && (!STATIC || lim < 32)) softmax_blocks<FP8, STATIC, true, 2>(w, pf, c, lim, lane);
   else softmax_blocks<FP8, STATIC, false, 2>(w, pf, c, lim, lane);
   if constexpr (LEAN) {
     bf16x8 vg[8];
@@ -577,7 +579,7 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     slot_prev = slot;                                                                                   \
     slot = slot == kRingT - 1 ? 0 : slot + 1;                                                           \
     const int tile = entry(i);                                                                          \
-    qk_tile<FP8, LEAN>(w, kbuf, kbuf + kKBytes, lane);                                                  \
+    qk_tile<FP8, LEAN, (MASKED) ? 2 : 4>(w, kbuf, kbuf + kKBytes, lane);                                \
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
     softmax_pv_tile<FP8, STATIC, LEAN, MASKED>(w, kbuf + kKBytes, ct, tail, lane);                      \
   }
@@ -709,10 +711,11 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     st2 = st2 == kStages2 - 1 ? 0 : st2 + 1;                                                            \
     if (it >= 2 * n_mine) continue; /* wave-uniform: this row-block has run out of tiles */             \
     const int tile = uniform_load(mine, it >> 1);                                                       \
-    qk_half<FP8>(w, hbuf, hbuf + kKHalf, lane);                                                         \
+    /* the running-max copy needs registers for the rescale: it takes the lean read-ahead (4 images) */ \
+    qk_half<FP8, !STATIC>(w, hbuf, hbuf + kKHalf, lane);                                                \
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
     const int lim = (tail && tile == nkt - 1) ? tail - 32 * (it & 1) : 32;                              \
-    softmax_pv_half<FP8, STATIC>(w, ct, lim, lane);                                                     \
+    softmax_pv_half<FP8, STATIC, !STATIC>(w, ct, lim, lane, hbuf + kKHalf);                             \
   }
     if (static_max) {
       PKH3_HALF_LOOP(true)
