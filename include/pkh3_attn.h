@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define PKH3_VERSION 102
+#define PKH3_VERSION 103
 
 enum {
   PKH3_OK = 0,
@@ -68,6 +68,12 @@ enum {
   PKH3_FLAG_KV_PREPARED = 1u << 2, /* K and V already lie in `workspace` as the attention kernel reads them, written
                                  there by pkh3_qkv_proj on the same stream with the same shapes and options: the
                                  call skips its own K/V pass; `k` and `v` are not read and may be NULL */
+  PKH3_FLAG_O_IMAGES = 1u << 3, /* `o` is not a [B, Sq, H, D] tensor but the operand-image buffer pkh3_out_proj reads
+                                 (what pkh3_pack_rows would make of the [Sq, H*D] output: pkh3_packed_bytes(Sq, H*D)
+                                 bytes, 16-byte aligned): the kernel's epilogue writes the images itself and the
+                                 separate packing pass disappears.  B must be 1; o_sb, o_ss, o_sh are not read.  Rows
+                                 of the buffer past ceil(Sq/32)*32 are left as they are (pkh3_out_proj never uses
+                                 what it computes from them) */
   PKH3_FLAG_LONG_KEY_KERNEL = 1u << 1 /* dense calls with at most 16 key tiles (Sk <= 1024) normally run a
                                  short-key form of the kernel (small workgroups, three per CU); this flag
                                  selects the long-key form for them too.  Same results to the tolerance of the

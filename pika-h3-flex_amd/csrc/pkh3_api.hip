@@ -50,10 +50,12 @@ int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = tru
   if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Sk < 1) return fail(PKH3_ESHAPE, "B, H, Sq, Sk must be >= 1");
   if (a->B > 65535 || a->H > 65535) return fail(PKH3_ESHAPE, "B and H must be <= 65535");
   if (a->Sq > (1 << 24) || a->Sk > (1 << 24)) return fail(PKH3_ESHAPE, "Sq and Sk must be <= 2^24");
-  if (a->flags & ~(uint32_t)(PKH3_FLAG_FP8_QK | PKH3_FLAG_LONG_KEY_KERNEL | PKH3_FLAG_KV_PREPARED))
+  if (a->flags & ~(uint32_t)(PKH3_FLAG_FP8_QK | PKH3_FLAG_LONG_KEY_KERNEL | PKH3_FLAG_KV_PREPARED | PKH3_FLAG_O_IMAGES))
     return fail(PKH3_EARG, "unknown flag bits 0x%x", a->flags);
   if ((a->flags & PKH3_FLAG_KV_PREPARED) && (a->key_mask || a->B != 1 || a->Sq != a->Sk))
     return fail(PKH3_EUNSUPPORTED, "prepared K/V (pkh3_qkv_proj) means one self-attention document: B = 1, Sq = Sk, no key mask");
+  if ((a->flags & PKH3_FLAG_O_IMAGES) && a->B != 1)
+    return fail(PKH3_EUNSUPPORTED, "output as operand images (PKH3_FLAG_O_IMAGES) means one document: B = 1");
   if (a->rope_mode < PKH3_ROPE_NONE || a->rope_mode > PKH3_ROPE_HALF) return fail(PKH3_EARG, "bad rope_mode %d", a->rope_mode);
   if (!(a->softmax_scale == a->softmax_scale) || isinf(a->softmax_scale)) return fail(PKH3_EARG, "softmax_scale is not finite");
   if ((a->q_norm_w || a->k_norm_w) && !(a->norm_eps >= 0.f)) return fail(PKH3_EARG, "norm_eps must be >= 0");
@@ -69,7 +71,12 @@ int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = tru
     if ((rc = check_tensor("k", a->k, a->k_sb, a->k_ss, a->k_sh, a->B, a->H))) return rc;
     if ((rc = check_tensor("v", a->v, a->v_sb, a->v_ss, a->v_sh, a->B, a->H))) return rc;
   }
-  if ((rc = check_tensor("o", a->o, a->o_sb, a->o_ss, a->o_sh, a->B, a->H))) return rc;
+  if (a->flags & PKH3_FLAG_O_IMAGES) {
+    if (!a->o) return fail(PKH3_ENULL, "o is NULL");
+    if (misaligned16(a->o)) return fail(PKH3_EALIGN, "o is not 16-byte aligned");
+  } else if ((rc = check_tensor("o", a->o, a->o_sb, a->o_ss, a->o_sh, a->B, a->H))) {
+    return rc;
+  }
   if (a->rope_mode != PKH3_ROPE_NONE) {
     if (!a->q_rope_cos || !a->q_rope_sin || !a->k_rope_cos || !a->k_rope_sin)
       return fail(PKH3_ENULL, "rope_mode set but a cos/sin table is NULL");
@@ -149,6 +156,9 @@ void build(const pkh3_attn_args* a, void* workspace, Launch& L) {
   f.kv = ws + L.w.kv_off; f.kv_bh_stride = k.out_bh_stride; f.kv_tile_stride = L.w.kvTileBytes;
   f.row_cnt = L.cnt;
   f.o = a->o; f.o_sb = a->o_sb; f.o_ss = a->o_ss; f.o_sh = a->o_sh;
+  // output as the operand images of the out-projection GEMM: [32-row block][(H*128)/16 k-steps] of 1 KiB
+  f.o_images = (a->flags & PKH3_FLAG_O_IMAGES) ? 1 : 0;
+  f.o_img_blk_stride = (int64_t)a->H * (kD / 16) * 1024;
   f.B = a->B; f.H = a->H; f.Sq = a->Sq; f.Sk = a->Sk; f.nQ64 = L.w.nQ64; f.nKt = L.w.nKt;
   const float scale = a->softmax_scale > 0.f ? a->softmax_scale : 1.0f / sqrtf((float)kD);
   f.c = scale * kLog2e;

@@ -756,6 +756,21 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
       }
   }
   // same wave wrote and reads: the LDS counter orders the two, no barrier
+  if (p.o_images) {
+    // operand images of the out-projection GEMM (32x32x16 form): image (row block q32, k-step h*8 + ks) holds, in lane
+    // (r = l % 32, hh = l / 32), elements 16*ks + 8*hh .. +7 of this head for row r -- one 1 KiB store per image
+    char* img = (char*)p.o + (int64_t)q32 * p.o_img_blk_stride + (int64_t)h * (kD / 16) * 1024;
+    const int r = lane & 31;
+    if (q32 * 32 >= p.Sq) return;  // a block without rows: the buffer may end before it
+    const bool live = q32 * 32 + r < p.Sq;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      bf16x8 v = *(const bf16x8*)(stage + r * 256 + (((2 * ks + hh) ^ (r & 15)) * 16));
+      if (!live) v = bf16x8{};
+      *(bf16x8*)(img + (ks * 64 + lane) * 16) = v;
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int row = 4 * i + (lane >> 4), c = lane & 15;

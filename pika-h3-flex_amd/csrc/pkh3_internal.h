@@ -68,6 +68,8 @@ struct FwdParams {
   const int* row_cnt;       // [B] valid keys after compaction, or null (= Sk)
   void* o;
   int64_t o_sb, o_ss, o_sh;
+  int o_images;             // write O as 32-row operand images [row block][H*8 k-steps] instead of [B, Sq, H, D] rows
+  int64_t o_img_blk_stride; // bytes between consecutive 32-row blocks of those images
   int B, H, Sq, Sk;
   int nQ64, nKt;
   float c;                  // softmax_scale * log2(e)

@@ -71,19 +71,26 @@ def fill_args(
     q, k, v, out, *, q_norm_weight=None, k_norm_weight=None, norm_eps=1e-6, rope_q=None, rope_k=None,
     rope_mode=_lib.ROPE_NONE, key_mask=None, block_mask: Optional[BlockMask] = None, fp8_qk=False,
     softmax_scale: Optional[float] = None, long_key_kernel: bool = False, kv_prepared: bool = False,
+    out_images: bool = False,
 ) -> Tuple[_lib.AttnArgs, list]:
     """Build ``pkh3_attn_args`` for these tensors.  Returns (args, keep_alive).  ``kv_prepared``: K and V
-    come from the fused projection (``pkh3_qkv_proj``) through the workspace; ``k`` and ``v`` are then None."""
+    come from the fused projection (``pkh3_qkv_proj``) through the workspace; ``k`` and ``v`` are then None.
+    ``out_images``: ``out`` is a uint8 operand-image buffer for ``pkh3_out_proj`` (``projections.packed_bytes(Sq,
+    H*D)`` bytes) instead of a ``[B, Sq, H, D]`` tensor, and B must be 1."""
     if kv_prepared != (k is None) or (k is None) != (v is None):
         raise ValueError("k and v are None exactly when kv_prepared is set")
-    for n, t in (("q", q), ("k", k), ("v", v), ("out", out)):
+    for n, t in (("q", q), ("k", k), ("v", v)) + (() if out_images else (("out", out),)):
         if t is not None:
             _check_bshd(n, t)
     B, Sq, H, D = q.shape
     Sk = Sq if k is None else k.shape[1]
     if k is not None and (tuple(k.shape) != (B, Sk, H, D) or tuple(v.shape) != (B, Sk, H, D)):
         raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
-    if tuple(out.shape) != (B, Sq, H, D):
+    if out_images:
+        need = ((Sq + 255) // 256 * 256) * H * D * 2
+        if out.dtype != torch.uint8 or not out.is_contiguous() or out.numel() < need or B != 1:
+            raise ValueError(f"out_images: out must be a contiguous uint8 buffer of at least {need} bytes and B must be 1")
+    elif tuple(out.shape) != (B, Sq, H, D):
         raise ValueError(f"out shape {tuple(out.shape)} != {(B, Sq, H, D)}")
     dev = q.device
     for n, t in (("k", k), ("v", v), ("out", out)):
@@ -97,7 +104,8 @@ def fill_args(
         a.k, a.v = k.data_ptr(), v.data_ptr()
         a.k_sb, a.k_ss, a.k_sh = k.stride(0), k.stride(1), k.stride(2)
         a.v_sb, a.v_ss, a.v_sh = v.stride(0), v.stride(1), v.stride(2)
-    a.o_sb, a.o_ss, a.o_sh = out.stride(0), out.stride(1), out.stride(2)
+    if not out_images:
+        a.o_sb, a.o_ss, a.o_sh = out.stride(0), out.stride(1), out.stride(2)
     a.B, a.H, a.Sq, a.Sk, a.D = B, H, Sq, Sk, D
     a.softmax_scale = float(softmax_scale) if softmax_scale is not None else 0.0
     qw = _f32("q_norm_weight", q_norm_weight, (D,), dev)
@@ -137,7 +145,7 @@ def fill_args(
         a.blk_row_ptr, a.blk_col_idx = block_mask.row_ptr.data_ptr(), block_mask.col_idx.data_ptr()
         keep += [block_mask.row_ptr, block_mask.col_idx]
     a.flags = ((_lib.FLAG_FP8_QK if fp8_qk else 0) | (_lib.FLAG_LONG_KEY_KERNEL if long_key_kernel else 0)
-               | (_lib.FLAG_KV_PREPARED if kv_prepared else 0))
+               | (_lib.FLAG_KV_PREPARED if kv_prepared else 0) | (_lib.FLAG_O_IMAGES if out_images else 0))
     keep += [qw, kw]
     return a, keep
 
@@ -162,6 +170,8 @@ def attention(
     Runs asynchronously on the current stream and returns ``out`` ([B, Sq, H, D], bf16)."""
     lib = _lib.load()
     if out is None:
+        if opts.get("out_images"):
+            raise ValueError("out_images needs the image buffer as out")
         out = torch.empty((q.shape[0], q.shape[1], q.shape[2], q.shape[3]), dtype=torch.bfloat16, device=q.device)
     args, keep = fill_args(q, k, v, out, **opts)
     if static_scratch:

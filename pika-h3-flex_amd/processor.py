@@ -228,11 +228,12 @@ class PikaH3AttnProcessor:
             rope_cos_sin = self._tables(position_ids, rope_key)
         if rope_cos_sin is not None:
             opts.update(rope_mode=self.rope_mode, rope_q=rope_cos_sin, rope_k=rope_cos_sin)
-        o = qkv_attention(x_img, S, packed["q"], packed["k"], packed["v"], heads=H, **opts)
+        # the attention kernel writes its output as the operand images of the out-projection: no packing pass
+        o_img = qkv_attention(x_img, S, packed["q"], packed["k"], packed["v"], heads=H, out_images=True, **opts)
         res = None
         if residual is not None:
             res = residual[0] if residual.dim() == 3 else residual
             if res.dtype != torch.bfloat16:
                 res = res.to(torch.bfloat16)
-        y = out_proj(o.view(S, C), packed["out"], gate=gate, row_index=gate_index, residual=res)
+        y = out_proj(None, packed["out"], gate=gate, row_index=gate_index, residual=res, o_img=o_img, rows=S)
         return y.view(1, S, C).to(hidden_states.dtype)

@@ -153,7 +153,9 @@ def qkv_attention(x_img: torch.Tensor, S: int, q: PackedLinear, k: PackedLinear,
     """One self-attention call from packed activations: ``to_q / to_k / to_v`` (+ adapters) with the K side's
     norm + rotation (+ fp8 quantisation) and the K/V layout in the GEMM epilogue, then the attention kernel on
     what the GEMM left in the workspace.  ``opts`` are those of :func:`ops.fill_args` (norm weights, rope
-    tables, ``fp8_qk``, ``block_mask`` ...).  Returns O ``[1, S, H, D]`` bf16 (and Q when ``return_q``)."""
+    tables, ``fp8_qk``, ``block_mask`` ...).  Returns O ``[1, S, H, D]`` bf16 (and Q when ``return_q``); with
+    ``out_images=True`` O comes back as the packed operand images :func:`out_proj` takes (``o_img=``), written
+    by the attention kernel itself."""
     lib = _lib.load()
     dev = x_img.device
     K = q.K
@@ -164,7 +166,8 @@ def qkv_attention(x_img: torch.Tensor, S: int, q: PackedLinear, k: PackedLinear,
         raise ValueError("x_img is not a packed [S, K] activation buffer")
     qt = torch.empty((1, S, heads, HEAD_DIM), dtype=torch.bfloat16, device=dev)
     if out is None:
-        out = torch.empty_like(qt)
+        out = (torch.empty(packed_bytes(S, heads * HEAD_DIM), dtype=torch.uint8, device=dev) if opts.get("out_images")
+               else torch.empty_like(qt))
     args, keep = fill_args(qt, None, None, out, kv_prepared=True, **opts)
     ws = torch.empty(workspace_bytes(args), dtype=torch.uint8, device=dev)
     args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
@@ -185,17 +188,29 @@ def qkv_attention(x_img: torch.Tensor, S: int, q: PackedLinear, k: PackedLinear,
     return (out, qt) if return_q else out
 
 
-def out_proj(o: torch.Tensor, proj: PackedLinear, *, gate: Optional[torch.Tensor] = None,
-             row_index: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+def out_proj(o: Optional[torch.Tensor], proj: PackedLinear, *, gate: Optional[torch.Tensor] = None,
+             row_index: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None,
+             o_img: Optional[torch.Tensor] = None, rows: Optional[int] = None) -> torch.Tensor:
     """``residual + gate[row_index] * (o W^T + bias + adapter)`` for the attention output ``o`` bf16 ``[S, K]``
-    (e.g. ``O.view(S, H*D)``).  ``gate`` bf16 ``[table rows, N]``, ``residual`` bf16 ``[S, N]``."""
+    (e.g. ``O.view(S, H*D)``).  ``gate`` bf16 ``[table rows, N]``, ``residual`` bf16 ``[S, N]``.  Instead of ``o``
+    the packed images of ``rows`` output rows can be given (``o_img``, from ``qkv_attention(..., out_images=True)``)."""
     lib = _lib.load()
-    o = _rows_bf16("o", o)
-    S, K = o.shape
-    if K != proj.K:
-        raise ValueError(f"o has {K} columns, the projection expects {proj.K}")
-    dev = o.device
-    o_img = pack_rows(o)
+    if (o is None) == (o_img is None):
+        raise ValueError("give either o or o_img")
+    if o_img is not None:
+        if rows is None or rows < 1:
+            raise ValueError("o_img needs the number of rows")
+        S, K = int(rows), proj.K
+        if o_img.dtype != torch.uint8 or not o_img.is_contiguous() or o_img.numel() < packed_bytes(S, K):
+            raise ValueError("o_img is not a packed [rows, K] activation buffer")
+        dev = o_img.device
+    else:
+        o = _rows_bf16("o", o)
+        S, K = o.shape
+        if K != proj.K:
+            raise ValueError(f"o has {K} columns, the projection expects {proj.K}")
+        dev = o.device
+        o_img = pack_rows(o)
     y = torch.empty((S, proj.N), dtype=torch.bfloat16, device=dev)
     a = _lib.OutArgs()
     a.o_img, a.S, a.K, a.N = o_img.data_ptr(), S, K, proj.N

@@ -22,7 +22,7 @@ def test_header_symbols_are_exported(lib):
 
 
 def test_version_and_strerror(lib):
-    assert lib.pkh3_version() == 102
+    assert lib.pkh3_version() == 103
     assert lib.pkh3_strerror(0) == b"ok"
     assert b"128" in lib.pkh3_strerror(_lib.PKH3_EHEADDIM)
 
@@ -88,6 +88,10 @@ def test_workspace_bytes_host_only(lib):
      _lib.PKH3_EUNSUPPORTED),
     (lambda a: (setattr(a, "flags", 1), setattr(a, "key_mask", 0x40000)), _lib.PKH3_EUNSUPPORTED),
     (lambda a: setattr(a, "softmax_scale", float("nan")), _lib.PKH3_EARG),
+    # output as operand images: one document only; the strides are not looked at, the pointer is
+    (lambda a: (setattr(a, "flags", _lib.FLAG_O_IMAGES), setattr(a, "B", 2)), _lib.PKH3_EUNSUPPORTED),
+    (lambda a: (setattr(a, "flags", _lib.FLAG_O_IMAGES), setattr(a, "o", 0)), _lib.PKH3_ENULL),
+    (lambda a: (setattr(a, "flags", _lib.FLAG_O_IMAGES), setattr(a, "o", 0x10008)), _lib.PKH3_EALIGN),
 ])
 def test_argument_errors_are_reported_before_any_launch(lib, mutate, code):
     a = _valid_args()

@@ -373,3 +373,37 @@ def test_document_kwargs_drive_the_fused_block():
     # the keyframe rows and the frame they pin share a grid, so with equal inputs they would rotate alike: spot-check the layout
     vi = mi["video_indices"]
     assert torch.equal(pos[vi[:60], 1:], pos[vi[60:120], 1:]) and float(pos[vi[:60], 0].abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("S,H,variant", [(300, 2, "dense"), (1000, 3, "fp8"), (777, 2, "sparse"), (130, 1, "short")])
+def test_attention_writes_the_out_projection_images(S, H, variant):
+    """With PKH3_FLAG_O_IMAGES the attention epilogue writes what pkh3_pack_rows would make of its row-major output:
+    the same bytes for every image row that exists, in every form of the kernel (long, short-key, split, block-sparse)."""
+    import pika_h3_flex_amd as pk
+    from pika_h3_flex_amd import projections as P
+
+    g = torch.Generator().manual_seed(21)
+    q, k, v = (torch.randn((1, S, H, 128), generator=g).to(torch.bfloat16).cuda() for _ in range(3))
+    w = (1.0 + 0.1 * torch.randn(128, generator=g)).cuda()
+    pos = (torch.rand((S, 3), generator=g, dtype=torch.float64) * 20).cuda()
+    opts = dict(q_norm_weight=w, k_norm_weight=w, rope_mode=pk.ROPE_INTERLEAVED, rope_q=pk.rope_tables(pos))
+    if variant == "fp8":
+        opts["fp8_qk"] = True
+    if variant == "sparse":
+        nt = (S + 63) // 64
+        keep = torch.rand((nt, nt), generator=g) < 0.5
+        keep |= torch.eye(nt, dtype=torch.bool)
+        opts["block_mask"] = pk.BlockMask.from_dense(keep.cuda())
+    if variant != "short":
+        opts["long_key_kernel"] = variant == "dense"
+    rows = pk.attention(q, k, v, **opts)
+    want = P.pack_rows(rows.view(S, H * 128))
+    img = torch.full((P.packed_bytes(S, H * 128),), 0xAB, dtype=torch.uint8, device="cuda")
+    got = pk.attention(q, k, v, out=img, out_images=True, **opts)
+    torch.cuda.synchronize()
+    assert got is img
+    live = ((S + 31) // 32) * (H * 128 // 16) * 1024            # bytes of the 32-row blocks that hold rows
+    assert torch.equal(img[:live], want[:live])
+    assert bool((img[live:] == 0xAB).all())                     # blocks past the last row are left alone
+    with pytest.raises(ValueError):
+        pk.attention(q.expand(2, -1, -1, -1), k.expand(2, -1, -1, -1), v.expand(2, -1, -1, -1), out=img, out_images=True, **opts)
