@@ -21,6 +21,8 @@
 // head) x tokens tq*64..+63 (one K/V tile): 8 accumulators of 32x32.  Per 32-wide k-chunk a wave reads 8 weight
 // and 4 activation images for 16 MFMAs.  LoRA is a second K segment: k-chunks beyond the hidden size take their
 // activation images from the down-projected rows (x A^T, scaled) and their weight images from B.
+#include <type_traits>
+
 #include "pkh3_common.h"
 #include "pkh3_internal.h"
 
@@ -74,17 +76,19 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
   const char* seg2 = w_side ? tg.w2_img + (int64_t)(n_tile_in_target * 8 + blk0) * tg.w2_blk_stride
                             : tg.a2_img + (int64_t)(m_tile * 8 + blk0) * tg.a2_blk_stride;
   const int64_t seg2_step = w_side ? tg.w2_blk_stride : tg.a2_blk_stride;
-  auto dma = [&](int kc, int slot) {
+  // this wave's copies of one chunk: PP pieces of 1 KiB from `g` (two consecutive k-step images of one block are
+  // contiguous, 2 KiB; the next block is `step` bytes on) into ring slot `slot`
+  auto dma_from = [&](const char* g, int64_t step, int slot) {
     char* d = lds_raw + slot * kGemmStageBytes + piece0 * 1024;
-    const bool first = kc < nk1;
-    const char* g = first ? seg1 + (int64_t)kc * 2048 : seg2 + (int64_t)(kc - nk1) * 2048;
-    const int64_t step = first ? seg1_step : seg2_step;
-    // two consecutive k-step images of one block are contiguous (2 KiB); the next block is `step` bytes on
 #pragma unroll
     for (int b = 0; b < PP / 2; ++b) {
       gemm_dma16(g + b * step, lane_off, d + b * 2048);
       gemm_dma16(g + b * step + 1024, lane_off, d + b * 2048 + 1024);
     }
+  };
+  auto dma = [&](int kc, int slot) {
+    const bool first = kc < nk1;
+    dma_from(first ? seg1 + (int64_t)kc * 2048 : seg2 + (int64_t)(kc - nk1) * 2048, first ? seg1_step : seg2_step, slot);
   };
   // waits until at most `chunks` of this wave's newest chunk copies are still in flight
   auto wait_dma = [&](int chunks) {
@@ -130,23 +134,55 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
   };
   if (head_live) read_frags(0, 0, wf[0], xf[0]);
   int slot = 0;
-  for (int kc = 0; kc < nk; ++kc) {
-    if (kc + 1 < nk) {
+  // source of the next chunk to copy (chunk kc + 3 in the steady loop): a running pointer inside its K segment
+  const char* g_next = nullptr;
+  int64_t step_next = seg1_step;
+  int left_next = 0;  // chunks left in the segment g_next walks, this one included
+  if (nk > 3) {
+    const bool first = 3 < nk1;
+    g_next = first ? seg1 + 3 * 2048 : seg2 + (int64_t)(3 - nk1) * 2048;
+    step_next = first ? seg1_step : seg2_step;
+    left_next = first ? nk1 - 3 : nk - 3;
+  }
+  // One chunk.  MORE1/2/3: chunks kc+1 / kc+2 / kc+3 exist (compile-time, so the steady loop carries no tests).
+  auto chunk = [&](auto more1, auto more2, auto more3) {
+    if constexpr (more1()) {
       // chunk kc+1 has landed (this wave's pieces; the barrier covers the others'); only chunk kc+2's copies may be pending
-      if (kc + 2 < nk) wait_dma(1);
+      if constexpr (more2()) wait_dma(1);
       else wait_dma(0);
       __syncthreads();
-      if (kc + 3 < nk) dma(kc + 3, (slot + 3) & 3);
     }
     const int next = (slot + 1) & 3;
     if (head_live) {  // wave-uniform: a head past the end of the target only copies and synchronises
       read_frags(slot, 1, wf[1], xf[1]);
       mfmas(wf[0], xf[0]);
-      if (kc + 1 < nk) read_frags(next, 0, wf[0], xf[0]);
+    }
+    // the copies of chunk kc+3 are issued under the first k-step's MFMAs, not in front of them: their address
+    // arithmetic is a scalar chain every wave of the workgroup would otherwise run at the same time, right after
+    // the barrier, with the MFMA pipe idle
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (more3()) {
+      dma_from(g_next, step_next, (slot + 3) & 3);
+      g_next += 2048;
+      if (--left_next == 0) {
+        g_next = seg2;
+        step_next = seg2_step;
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (head_live) {
+      if constexpr (more1()) read_frags(next, 0, wf[0], xf[0]);
       mfmas(wf[1], xf[1]);
     }
     slot = next;
-  }
+  };
+  constexpr std::true_type yes{};
+  constexpr std::false_type no{};
+  int kc = 0;
+  for (; kc + 3 < nk; ++kc) chunk(yes, yes, yes);
+  if (kc + 2 < nk) { chunk(yes, yes, no); ++kc; }
+  if (kc + 1 < nk) { chunk(yes, no, no); ++kc; }
+  chunk(no, no, no);
   // let the last MFMA retire before anything the compiler places after the loop reads the accumulators
 #pragma unroll
   for (int t2 = 0; t2 < TB; ++t2)
