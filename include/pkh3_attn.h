@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define PKH3_VERSION 103
+#define PKH3_VERSION 104
 
 enum {
   PKH3_OK = 0,
@@ -150,8 +150,8 @@ int pkh3_rope_tables(const double* position_ids, int32_t S, const int32_t axis_d
  * modulation that feeds them (patches/0001-h3-adaln-fp32.patch:34-40: norm(x) * (1 + scale[idx]) +
  * shift[idx], rows gathered by `timestep_indices`, src/pika_h3/core/wrapper.py:182-190,196-197).
  *
- * Matrix operands are kept as "operand images": 1 KiB blocks of 32 rows x 16 contraction elements in
- * the register order of the gfx950 32x32x16 MFMA.  Weights are packed once (pkh3_pack_weight) when
+ * Matrix operands are kept as "operand images": 1 KiB blocks of 16 rows x 32 contraction elements in
+ * the register order of the gfx950 16x16x32 MFMA.  Weights are packed once (pkh3_pack_weight) when
  * they are loaded; activations are packed by the kernel that produces them (pkh3_adaln_modulate) or
  * by pkh3_pack_rows.  A packed buffer for [rows, K] takes pkh3_packed_bytes(rows, K) bytes, 256-byte
  * aligned; rows are padded to a multiple of 256 with zeros.  K must be a multiple of 32 and <= 4096.

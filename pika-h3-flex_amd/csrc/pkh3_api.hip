@@ -156,9 +156,9 @@ void build(const pkh3_attn_args* a, void* workspace, Launch& L) {
   f.kv = ws + L.w.kv_off; f.kv_bh_stride = k.out_bh_stride; f.kv_tile_stride = L.w.kvTileBytes;
   f.row_cnt = L.cnt;
   f.o = a->o; f.o_sb = a->o_sb; f.o_ss = a->o_ss; f.o_sh = a->o_sh;
-  // output as the operand images of the out-projection GEMM: [32-row block][(H*128)/16 k-steps] of 1 KiB
+  // output as the operand images of the out-projection GEMM: [16-row block][(H*128)/32 k-steps] of 1 KiB
   f.o_images = (a->flags & PKH3_FLAG_O_IMAGES) ? 1 : 0;
-  f.o_img_blk_stride = (int64_t)a->H * (kD / 16) * 1024;
+  f.o_img_blk_stride = (int64_t)a->H * (kD / 32) * 1024;
   f.B = a->B; f.H = a->H; f.Sq = a->Sq; f.Sk = a->Sk; f.nQ64 = L.w.nQ64; f.nKt = L.w.nKt;
   const float scale = a->softmax_scale > 0.f ? a->softmax_scale : 1.0f / sqrtf((float)kD);
   f.c = scale * kLog2e;
@@ -209,7 +209,7 @@ int run_pack(const void* x, int64_t row_stride, int32_t rows, int32_t K, int hea
   PackParams p{};
   p.x = x; p.row_stride = row_stride; p.rows = rows; p.rows_padded = (int)padded_rows(rows); p.K = K;
   p.head_perm = head_perm; p.norm = norm; p.eps = eps; p.shift = shift; p.scale = scale; p.table_stride = table_stride;
-  p.row_index = row_index; p.out = (char*)out; p.out_blk_stride = (int64_t)(K / 16) * 1024;
+  p.row_index = row_index; p.out = (char*)out; p.out_blk_stride = (int64_t)(K / 32) * 1024;
   hipError_t e = launch_pack_rows(p, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "pack_rows");
   g_err[0] = 0;
@@ -433,8 +433,8 @@ int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream)
   hipError_t e;
   const int H = a->H, N = H * kD;
   const bool fp8 = a->flags & PKH3_FLAG_FP8_QK;
-  const int64_t w_blk = (int64_t)(p->K / 16) * 1024;       // bytes of one 32-row block of images over K
-  const int64_t b_blk = (int64_t)(PKH3_LORA_RANK / 16) * 1024;
+  const int64_t w_blk = (int64_t)(p->K / 32) * 1024;       // bytes of one 16-row block of images over K
+  const int64_t b_blk = (int64_t)(PKH3_LORA_RANK / 32) * 1024;
   const int64_t xa_blk = 3 * b_blk;                        // down-projected rows: three targets side by side
   const int m_tiles = (int)(padded_rows(p->S) / 256);
 
@@ -453,7 +453,7 @@ int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream)
       tg.w_img = (const char*)lin[t]->lora_a_img; tg.w_blk_stride = w_blk;
       tg.out_scale = lin[t]->lora_scale;
       tg.out = (char*)p->lora_workspace + t * b_blk; tg.out_head_stride = 0;
-      tg.out_blk_stride = 2 * xa_blk; tg.out_sub_stride = (int)xa_blk;
+      tg.out_blk_stride = xa_blk;
       tg.rope_mode = PKH3_ROPE_NONE;
       g.n_tiles += 1;
     }
@@ -480,7 +480,6 @@ int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream)
     q.epi = kEpiRows; q.out = (char*)a->q; q.out_row_stride = a->q_ss; q.out_head_elems = (int)a->q_sh;
     GemmTarget& k = g.tg[1];
     k.epi = kEpiKImg; k.out = L.kp.out; k.out_head_stride = L.kp.out_bh_stride; k.out_blk_stride = L.kp.out_blk_stride;
-    k.out_sub_stride = fp8 ? kK8TileBytes / 2 : kKTileBytes / 2;
     k.norm_w = a->k_norm_w; k.norm_eps = a->norm_eps; k.rope_mode = a->rope_mode; k.cos_t = a->k_rope_cos; k.sin_t = a->k_rope_sin;
     k.norm_max = L.kp.norm_max; k.fp8 = fp8; k.scale_out = L.kp.scale_out; k.scale_head_stride = L.w.nKt;
     GemmTarget& v = g.tg[2];
@@ -512,8 +511,8 @@ int pkh3_out_proj(const pkh3_out_args* p, void* stream) {
     return fail(PKH3_EWORKSPACE, "out_proj: lora_workspace missing, misaligned (256 B) or smaller than %zu bytes", lora_need);
   hipStream_t st = (hipStream_t)stream;
   hipError_t e;
-  const int64_t w_blk = (int64_t)(p->K / 16) * 1024;
-  const int64_t b_blk = (int64_t)(PKH3_LORA_RANK / 16) * 1024;
+  const int64_t w_blk = (int64_t)(p->K / 32) * 1024;
+  const int64_t b_blk = (int64_t)(PKH3_LORA_RANK / 32) * 1024;
   const int m_tiles = (int)(padded_rows(p->S) / 256);
   if (lora) {
     GemmParams g{};
@@ -523,7 +522,7 @@ int pkh3_out_proj(const pkh3_out_args* p, void* stream) {
     tg = GemmTarget{};
     tg.epi = kEpiAImg; tg.n = PKH3_LORA_RANK; tg.n_tiles = 1;
     tg.w_img = (const char*)p->proj.lora_a_img; tg.w_blk_stride = w_blk; tg.out_scale = p->proj.lora_scale;
-    tg.out = (char*)p->lora_workspace; tg.out_blk_stride = 2 * b_blk; tg.out_sub_stride = (int)b_blk;
+    tg.out = (char*)p->lora_workspace; tg.out_blk_stride = b_blk;
     if ((e = launch_gemm(g, st)) != hipSuccess) return hip_fail(e, "lora down-projection");
   }
   GemmParams g{};

@@ -757,17 +757,21 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   }
   // same wave wrote and reads: the LDS counter orders the two, no barrier
   if (p.o_images) {
-    // operand images of the out-projection GEMM (32x32x16 form): image (row block q32, k-step h*8 + ks) holds, in lane
-    // (r = l % 32, hh = l / 32), elements 16*ks + 8*hh .. +7 of this head for row r -- one 1 KiB store per image
-    char* img = (char*)p.o + (int64_t)q32 * p.o_img_blk_stride + (int64_t)h * (kD / 16) * 1024;
-    const int r = lane & 31;
+    // operand images of the out-projection GEMM: image (16-row block, k-step h*4 + ks) holds, in lane (c = l % 16,
+    // g = l / 16), elements 32*ks + 8*g .. +7 of this head for row c of the block -- one 1 KiB store per image
     if (q32 * 32 >= p.Sq) return;  // a block without rows: the buffer may end before it
-    const bool live = q32 * 32 + r < p.Sq;
+    const int c16 = lane & 15, g4 = lane >> 4;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      bf16x8 v = *(const bf16x8*)(stage + r * 256 + (((2 * ks + hh) ^ (r & 15)) * 16));
-      if (!live) v = bf16x8{};
-      *(bf16x8*)(img + (ks * 64 + lane) * 16) = v;
+    for (int rb = 0; rb < 2; ++rb) {
+      const int r = 16 * rb + c16;
+      const bool live = q32 * 32 + r < p.Sq;
+      char* img = (char*)p.o + (int64_t)(q32 * 2 + rb) * p.o_img_blk_stride + (int64_t)h * (kD / 32) * 1024;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        bf16x8 v = *(const bf16x8*)(stage + r * 256 + (((4 * ks + g4) ^ (r & 15)) * 16));
+        if (!live) v = bf16x8{};
+        *(bf16x8*)(img + (ks * 64 + lane) * 16) = v;
+      }
     }
     return;
   }

@@ -1,25 +1,26 @@
-// Projection GEMMs around the attention kernel (gfx950, bf16 MFMA 32x32x16, fp32 accumulation):
+// Projection GEMMs around the attention kernel (gfx950, bf16 MFMA 16x16x32, fp32 accumulation):
 //   to_q / to_k / to_v  (+ LoRA)  from the modulated hidden states, with the K side's RMSNorm + rotation
 //                       (+ fp8 quantisation) and the K / V operand-image layout done in the epilogue, so that
 //                       K and V go from the accumulators straight into the records the attention kernel reads
 //   to_out.0 (+ LoRA)   from the attention output, with bias, per-row gate and residual in the epilogue
 //   LoRA down-projection x A^T, written as operand images for the second K segment of the GEMMs above
 //
-// Operands.  Both operands come as 1 KiB operand images (32 rows x 16 contraction elements, lane l holds row
-// l%32, elements 8*(l/32)..+7): activations as [token block][k-step], weights as [feature block][k-step] (packed
-// once when the weights are loaded).  They move HBM/L2 -> LDS -> VGPR as straight 16-byte copies, like the K/V
-// tiles of the attention kernel: direct-to-LDS loads into a 4-slot ring, three chunks ahead, one barrier per chunk.
-// Since the two MFMA operands have the same register form, one pair of images serves both orientations:
+// Operands.  Both operands come as 1 KiB operand images (16 rows x 32 contraction elements, lane l holds row
+// l%16, elements 8*(l/16)..+7 -- the shape of the attention kernel's K images): activations as [16-token
+// block][k-step], weights as [16-feature block][k-step] (packed once when the weights are loaded).  They move
+// HBM/L2 -> LDS -> VGPR as straight 16-byte copies, like the K/V tiles of the attention kernel: direct-to-LDS loads
+// into a 4-slot ring, three chunks ahead, one barrier per chunk.  Since the two MFMA operands have the same register
+// form, one pair of images serves both orientations:
 //   C^T = W x^T  (features down the accumulator registers, one token per lane)   Q, K, row-major outputs
 //   C   = x W^T  (tokens down the registers, one feature per lane)               V images
-// Weight rows are stored permuted inside each 128-feature head so that, in the C^T form, the 64 accumulator
-// values of a lane are exactly the 64 head-dim elements d = 16*ks + 8*hh + j the row transform
-// (norm_rope_row) works on: whole 8-element pieces of the row, which the epilogue stores at their places in the
-// attention kernel's K tile (a different image shape: that kernel runs on the 16x16 MFMAs, these GEMMs on 32x32).
+// Weight rows are stored permuted inside each 128-feature head so that, in the C^T form, the 32 accumulator
+// values a lane holds for a token are the four 8-element pieces p8 = 4*ks + g (elements 32*ks + 8*g .. +7) of that
+// token's head row: exactly what lane (g, c) of the attention kernel's K images carries, so the K epilogue stores
+// its accumulators (after norm and rotation) without any lane movement, and so do the row-major and the V epilogues.
 //
 // Work split.  Workgroup = 8 waves = 256 tokens x 256 features; wave (fh, tq) owns features fh*128..+127 (one
-// head) x tokens tq*64..+63 (one K/V tile): 8 accumulators of 32x32.  Per 32-wide k-chunk a wave reads 8 weight
-// and 4 activation images for 16 MFMAs.  LoRA is a second K segment: k-chunks beyond the hidden size take their
+// head) x tokens tq*64..+63 (one K/V tile): 32 accumulators of 16x16.  Per 32-wide k-chunk a wave reads 8 weight
+// and 4 activation images for 32 MFMAs.  LoRA is a second K segment: k-chunks beyond the hidden size take their
 // activation images from the down-projected rows (x A^T, scaled) and their weight images from B.
 #include <type_traits>
 
@@ -30,7 +31,7 @@ namespace pkh3 {
 
 constexpr int kGemmWaves = 8;
 constexpr int kGemmTile = 256;                      // tokens and features per workgroup
-constexpr int kGemmChunkK = 32;                     // contraction elements per ring slot
+constexpr int kGemmChunkK = 32;                     // contraction elements per ring slot = one k-step
 constexpr int kGemmStageBytes = 2 * kGemmTile * kGemmChunkK * 2;  // weight part + activation part
 constexpr int kGemmRing = 4;
 
@@ -43,52 +44,105 @@ __device__ __forceinline__ void gemm_dma16(const char* g, unsigned lane_off, cha
                : "memory", "m0");
 }
 
-// In the C^T form, accumulator value (db, i) of a lane with half hh is head-dim element
-// 16 * (2*db + (i >> 3)) + 8*hh + (i & 7) of the lane's token: element (ks, j) = (2*db + (i >> 3), i & 7) of the
-// lane's row in the layout of norm_rope_row, i.e. index 16*db + i of its x[64] (see pack_rows_kernel for the
-// weight-row permutation that makes it so).
+// RMSNorm + rotation of a quarter row: lane group g of a token holds the pieces p8 = 4*ks + g, i.e. elements
+// d = 32*ks + 8*g + j at x[8*ks + j]; the three other lane groups (lanes l ^ 16, l ^ 32, l ^ 48) hold the rest of the
+// row, so the sum of squares needs two exchanges and both pairings of the rotation (interleaved (2i, 2i+1) /
+// half-split (i, i+64): ks and ks + 2) stay inside the lane.  Same arithmetic as norm_rope_row.
+__device__ __forceinline__ void norm_rope_quarter(float (&x)[32], const RowTransform& t, int64_t table_row, bool valid, int g) {
+  if (t.norm_w) {
+    float ssq = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) ssq += x[i] * x[i];
+    ssq = wave_sum_groups(ssq);
+    const float ms = ssq * (1.0f / kD) + t.eps;
+    const float rs = ms > 0.f ? rsqrtf(ms) : 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const f32x4 w0 = *(const f32x4*)(t.norm_w + 32 * ks + 8 * g), w1 = *(const f32x4*)(t.norm_w + 32 * ks + 8 * g + 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[ks * 8 + j] *= rs * w0[j];
+        x[ks * 8 + 4 + j] *= rs * w1[j];
+      }
+    }
+  }
+  if (t.rope_mode == 1 && valid) {
+    const float* ct = t.cos_t + table_row * (kD / 2);
+    const float* st = t.sin_t + table_row * (kD / 2);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const f32x4 c = *(const f32x4*)(ct + 16 * ks + 4 * g), s = *(const f32x4*)(st + 16 * ks + 4 * g);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const float a0 = x[ks * 8 + 2 * jj], a1 = x[ks * 8 + 2 * jj + 1];
+        x[ks * 8 + 2 * jj] = a0 * c[jj] - a1 * s[jj];
+        x[ks * 8 + 2 * jj + 1] = a1 * c[jj] + a0 * s[jj];
+      }
+    }
+  } else if (t.rope_mode == 2 && valid) {
+    const float* ct = t.cos_t + table_row * (kD / 2);
+    const float* st = t.sin_t + table_row * (kD / 2);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const f32x4 c0 = *(const f32x4*)(ct + 32 * ks + 8 * g), c1 = *(const f32x4*)(ct + 32 * ks + 8 * g + 4);
+      const f32x4 s0 = *(const f32x4*)(st + 32 * ks + 8 * g), s1 = *(const f32x4*)(st + 32 * ks + 8 * g + 4);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float cj = j < 4 ? c0[j & 3] : c1[j & 3], sj = j < 4 ? s0[j & 3] : s1[j & 3];
+        const float lo = x[ks * 8 + j], hi = x[(ks + 2) * 8 + j];
+        x[ks * 8 + j] = lo * cj - hi * sj;
+        x[(ks + 2) * 8 + j] = hi * cj + lo * sj;
+      }
+    }
+  }
+}
 
-// WAVES = 8 (the form that ships): wave tile 128 features x 64 tokens, two waves per SIMD, accumulators in 128 VGPRs.
-// WAVES = 4 (wave tile 128 x 128, one wave per SIMD, 256 accumulator registers, half the LDS reads per MFMA) compiles
-// and passes the same tests but measured four times slower: with more than 256 registers the compiler moves
-// accumulators between the two register files inside the loop.
-template <int EPI, int WAVES>
+// eight values -> eight fp8 e4m3 bytes
+__device__ __forceinline__ i32x2 quant_fp8_piece(const float* x, float inv) {
+  i32x2 t;
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    int v = 0;
+    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * w] * inv, x[4 * w + 1] * inv, v, false);
+    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * w + 2] * inv, x[4 * w + 3] * inv, v, true);
+    t[w] = v;
+  }
+  return t;
+}
+
+template <int EPI>
 __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget& tg, int m_tile, int n_tile_in_target,
                                           char* lds_raw) {
-  constexpr int TB = 16 / WAVES;                     // 32-token blocks per wave
+  constexpr int WAVES = kGemmWaves;
   constexpr int PP = 32 / WAVES;                     // 1 KiB pieces of a chunk each wave copies
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int hh = lane >> 5, r = lane & 31;
-  const int fh = wave & 1, tq = wave >> 1;           // feature half (one head), token slice
+  const int g = lane >> 4, c = lane & 15;
+  const int fh = wave & 1, tq = wave >> 1;           // feature half (one head), 64-token slice
   const int head = n_tile_in_target * 2 + fh;        // 128-feature head inside the target
   const bool head_live = head * 128 < tg.n;
   const int nk1 = p.nk1, nk = p.nk1 + tg.nk2;
   const unsigned lane_off = lane * 16;
 
-  // this wave's 1 KiB pieces of every chunk: pieces PP*wave.. of [8 weight blocks x 2 k-steps | 8 token blocks x 2]
+  // this wave's 1 KiB pieces of every chunk: pieces PP*wave.. of [16 weight blocks | 16 token blocks]
   const int piece0 = wave * PP;
   const bool w_side = piece0 < 16;
-  const int blk0 = (piece0 & 15) >> 1;               // first of the 32-row blocks this wave copies
-  const char* seg1 = w_side ? tg.w_img + (int64_t)(n_tile_in_target * 8 + blk0) * tg.w_blk_stride
-                            : p.a_img + (int64_t)(m_tile * 8 + blk0) * p.a_blk_stride;
+  const int blk0 = piece0 & 15;                      // first of the 16-row blocks this wave copies
+  const char* seg1 = w_side ? tg.w_img + (int64_t)(n_tile_in_target * 16 + blk0) * tg.w_blk_stride
+                            : p.a_img + (int64_t)(m_tile * 16 + blk0) * p.a_blk_stride;
   const int64_t seg1_step = w_side ? tg.w_blk_stride : p.a_blk_stride;
-  const char* seg2 = w_side ? tg.w2_img + (int64_t)(n_tile_in_target * 8 + blk0) * tg.w2_blk_stride
-                            : tg.a2_img + (int64_t)(m_tile * 8 + blk0) * tg.a2_blk_stride;
+  const char* seg2 = w_side ? tg.w2_img + (int64_t)(n_tile_in_target * 16 + blk0) * tg.w2_blk_stride
+                            : tg.a2_img + (int64_t)(m_tile * 16 + blk0) * tg.a2_blk_stride;
   const int64_t seg2_step = w_side ? tg.w2_blk_stride : tg.a2_blk_stride;
-  // this wave's copies of one chunk: PP pieces of 1 KiB from `g` (two consecutive k-step images of one block are
-  // contiguous, 2 KiB; the next block is `step` bytes on) into ring slot `slot`
-  auto dma_from = [&](const char* g, int64_t step, int slot) {
+  // this wave's copies of one chunk: the chunk's image of PP consecutive blocks, `step` bytes apart, into ring slot `slot`
+  auto dma_from = [&](const char* gp, int64_t step, int slot) {
     char* d = lds_raw + slot * kGemmStageBytes + piece0 * 1024;
 #pragma unroll
-    for (int b = 0; b < PP / 2; ++b) {
-      gemm_dma16(g + b * step, lane_off, d + b * 2048);
-      gemm_dma16(g + b * step + 1024, lane_off, d + b * 2048 + 1024);
-    }
+    for (int b = 0; b < PP; ++b) gemm_dma16(gp + b * step, lane_off, d + b * 1024);
   };
   auto dma = [&](int kc, int slot) {
     const bool first = kc < nk1;
-    dma_from(first ? seg1 + (int64_t)kc * 2048 : seg2 + (int64_t)(kc - nk1) * 2048, first ? seg1_step : seg2_step, slot);
+    dma_from(first ? seg1 + (int64_t)kc * 1024 : seg2 + (int64_t)(kc - nk1) * 1024, first ? seg1_step : seg2_step, slot);
   };
   // waits until at most `chunks` of this wave's newest chunk copies are still in flight
   auto wait_dma = [&](int chunks) {
@@ -97,42 +151,44 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
 
-  f32x16 acc[TB][4];
+  f32x4 acc[4][8];                                   // (16-token block of the wave's 64, 16-feature block of the head)
 #pragma unroll
-  for (int t2 = 0; t2 < TB; ++t2)
+  for (int t = 0; t < 4; ++t)
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[t2][db][i] = 0.f;
+    for (int fb = 0; fb < 8; ++fb) acc[t][fb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // Ring of four chunks.  Entering iteration kc: chunk kc is in LDS for every wave and its first k-step's images are
-  // already on their way to this wave's registers; chunks kc+1 and kc+2 are in flight.  The barrier at the top makes
-  // chunk kc+1 visible and frees the slot of chunk kc-1 for chunk kc+3, so the first images of the next chunk can be
-  // read at the tail of this iteration and no wave starts a chunk by waiting for LDS.
+  // Ring of four chunks.  Entering iteration kc: chunk kc is in LDS for every wave and its token images and first four
+  // weight images are already on their way to this wave's registers; chunks kc+1 and kc+2 are in flight.  The barrier at
+  // the top makes chunk kc+1 visible and frees the slot of chunk kc-1 for chunk kc+3, so the first images of the next
+  // chunk can be read at the tail of this iteration and no wave starts a chunk by waiting for LDS.
   const int n_pre = nk < 3 ? nk : 3;
-  for (int c = 0; c < n_pre; ++c) dma(c, c);
+  for (int cc = 0; cc < n_pre; ++cc) dma(cc, cc);
   wait_dma(n_pre - 1);
   __syncthreads();
-  const int w_off = (fh * 4) * 2048 + lane * 16;            // weight blocks fh*4..+3 of a slot
-  const int a_off = 16384 + (tq * TB) * 2048 + lane * 16;   // this wave's token blocks
-  bf16x8 wf[2][4], xf[2][TB];
-  auto read_frags = [&](int slot, int ks, bf16x8 (&w4)[4], bf16x8 (&xt)[TB]) {
-    const char* base = lds_raw + slot * kGemmStageBytes + ks * 1024;
+  const int w_off = (fh * 8) * 1024 + lane * 16;            // weight blocks fh*8..+7 of a slot
+  const int a_off = 16384 + (tq * 4) * 1024 + lane * 16;    // this wave's token blocks
+  bf16x8 wa[4], wb[4], xc[4], xn[4];                        // weight blocks 0..3 / 4..7, token images of this / the next chunk
+  auto read_w = [&](int slot, int half, bf16x8 (&w4)[4]) {
 #pragma unroll
-    for (int db = 0; db < 4; ++db) w4[db] = *(const bf16x8*)(base + w_off + db * 2048);
-#pragma unroll
-    for (int t2 = 0; t2 < TB; ++t2) xt[t2] = *(const bf16x8*)(base + a_off + t2 * 2048);
+    for (int i = 0; i < 4; ++i) w4[i] = *(const bf16x8*)(lds_raw + slot * kGemmStageBytes + w_off + (half * 4 + i) * 1024);
   };
-  auto mfmas = [&](const bf16x8 (&w4)[4], const bf16x8 (&xt)[TB]) {
+  auto read_x = [&](int slot, bf16x8 (&x4)[4]) {
 #pragma unroll
-    for (int t2 = 0; t2 < TB; ++t2)
+    for (int t = 0; t < 4; ++t) x4[t] = *(const bf16x8*)(lds_raw + slot * kGemmStageBytes + a_off + t * 1024);
+  };
+  auto mfmas = [&](int half, const bf16x8 (&w4)[4], const bf16x8 (&x4)[4]) {
 #pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        if constexpr (EPI == kEpiVImg) acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xt[t2], w4[db], acc[t2][db], 0, 0, 0);
-        else acc[t2][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w4[db], xt[t2], acc[t2][db], 0, 0, 0);
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        if constexpr (EPI == kEpiVImg) acc[t][half * 4 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x4[t], w4[i], acc[t][half * 4 + i], 0, 0, 0);
+        else acc[t][half * 4 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w4[i], x4[t], acc[t][half * 4 + i], 0, 0, 0);
       }
   };
-  if (head_live) read_frags(0, 0, wf[0], xf[0]);
+  if (head_live) {
+    read_x(0, xc);
+    read_w(0, 0, wa);
+  }
   int slot = 0;
   // source of the next chunk to copy (chunk kc + 3 in the steady loop): a running pointer inside its K segment
   const char* g_next = nullptr;
@@ -140,7 +196,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
   int left_next = 0;  // chunks left in the segment g_next walks, this one included
   if (nk > 3) {
     const bool first = 3 < nk1;
-    g_next = first ? seg1 + 3 * 2048 : seg2 + (int64_t)(3 - nk1) * 2048;
+    g_next = first ? seg1 + 3 * 1024 : seg2 + (int64_t)(3 - nk1) * 1024;
     step_next = first ? seg1_step : seg2_step;
     left_next = first ? nk1 - 3 : nk - 3;
   }
@@ -154,16 +210,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
     }
     const int next = (slot + 1) & 3;
     if (head_live) {  // wave-uniform: a head past the end of the target only copies and synchronises
-      read_frags(slot, 1, wf[1], xf[1]);
-      mfmas(wf[0], xf[0]);
+      read_w(slot, 1, wb);
+      mfmas(0, wa, xc);
     }
-    // the copies of chunk kc+3 are issued under the first k-step's MFMAs, not in front of them: their address
+    // the copies of chunk kc+3 are issued under the first half's MFMAs, not in front of them: their address
     // arithmetic is a scalar chain every wave of the workgroup would otherwise run at the same time, right after
     // the barrier, with the MFMA pipe idle
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (more3()) {
       dma_from(g_next, step_next, (slot + 3) & 3);
-      g_next += 2048;
+      g_next += 1024;
       if (--left_next == 0) {
         g_next = seg2;
         step_next = seg2_step;
@@ -171,8 +227,15 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
     }
     __builtin_amdgcn_sched_barrier(0);
     if (head_live) {
-      if constexpr (more1()) read_frags(next, 0, wf[0], xf[0]);
-      mfmas(wf[1], xf[1]);
+      if constexpr (more1()) {
+        read_x(next, xn);
+        read_w(next, 0, wa);
+      }
+      mfmas(1, wb, xc);
+      if constexpr (more1()) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) xc[t] = xn[t];
+      }
     }
     slot = next;
   };
@@ -185,142 +248,149 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
   chunk(no, no, no);
   // let the last MFMA retire before anything the compiler places after the loop reads the accumulators
 #pragma unroll
-  for (int t2 = 0; t2 < TB; ++t2)
-    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc[t2][0]), "+v"(acc[t2][1]), "+v"(acc[t2][2]), "+v"(acc[t2][3])::"memory");
+  for (int t = 0; t < 4; ++t)
+    asm volatile("s_nop 15\n\ts_nop 15"
+                 : "+v"(acc[t][0]), "+v"(acc[t][1]), "+v"(acc[t][2]), "+v"(acc[t][3]), "+v"(acc[t][4]), "+v"(acc[t][5]),
+                   "+v"(acc[t][6]), "+v"(acc[t][7])::"memory");
   if (!head_live) return;
 
   const float* bias = tg.bias ? tg.bias + head * 128 : nullptr;
-  // the wave's token blocks, two at a time: one 64-token K/V tile per pair
-#pragma unroll
-  for (int tp = 0; tp < TB / 2; ++tp) {
-    const int tok0 = m_tile * kGemmTile + tq * (32 * TB) + tp * 64;
-    const int tile = m_tile * 4 + tq * (TB / 2) + tp;
-    if (tok0 >= p.M) break;                          // tiles past the last token: nothing to write
+  const int tok0 = m_tile * kGemmTile + tq * 64;     // the wave's 64 tokens: one K/V tile
+  const int tile = m_tile * 4 + tq;
+  if (tok0 >= p.M) return;                           // a tile past the last token: nothing to write
 
-    if constexpr (EPI == kEpiVImg) {
-      // lane = feature 32*db + r of the head, registers = tokens 8*(i/4) + 4*hh + i%4 of a 32-token block.  The V
-      // image (half = token block, db16) wants lane (g, c) = feature 16*db16 + c with tokens 16*(j/4) + 4*g + j%4:
-      // this lane's registers 4*(2*(j/4) + a) + j%4 are that piece for g = 2*a + hh, db16 = 2*db + r/16, c = r%16.
-      char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
+  if constexpr (EPI == kEpiVImg) {
+    // lane (g, c) = feature 16*fb + c of the head, registers = tokens 4*g + i of a 16-token block: the V image
+    // (half, db = fb) wants, in that same lane, the tokens 16*(j/4) + 4*g + j%4 of its 32: blocks 2*half and 2*half + 1
+    char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
 #pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2)
+    for (int half = 0; half < 2; ++half)
 #pragma unroll
-        for (int a = 0; a < 2; ++a)
+      for (int fb = 0; fb < 8; ++fb) {
+        const float bv = bias ? bias[16 * fb + c] : 0.f;
+        bf16x8 img;
 #pragma unroll
-          for (int db = 0; db < 4; ++db) {
-            const float bv = bias ? bias[32 * db + r] : 0.f;
-            bf16x8 img;
+        for (int j = 0; j < 8; ++j) {
+          const int token = tok0 + 32 * half + v_image_key(g, j);
+          img[j] = token < p.M ? (__bf16)(acc[2 * half + (j >> 2)][fb][j & 3] + bv) : (__bf16)0.0f;
+        }
+        *(bf16x8*)(rec + ((half * 8 + fb) * 64 + lane) * 16) = img;
+      }
+  } else {
+    // lane (g, c) = token 16*t + c; its accumulators (t, fb) are elements 32*ks + 8*g + j of the head row with
+    // fb = 2*ks + j/4, i = j%4 (the weight-row permutation, see pack_rows_kernel): x[8*ks + j]
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const int i = 4 * (2 * (j >> 2) + a) + (j & 3);
-              const int token = tok0 + 32 * t2 + 8 * (i >> 2) + 4 * hh + (i & 3);
-              img[j] = token < p.M ? (__bf16)(acc[2 * tp + t2][db][i] + bv) : (__bf16)0.0f;
-            }
-            *(bf16x8*)(rec + ((t2 * 8 + 2 * db + (r >> 4)) * 64 + 16 * (2 * a + hh) + (r & 15)) * 16) = img;
-          }
-    } else {
-      // lane = token, its 64 accumulator values per token block = head-dim elements 16*ks + 8*hh + j in x[ks*8 + j]
-      float x[2][64];
+    for (int t = 0; t < 4; ++t) {
+      const int token = tok0 + 16 * t + c;
+      const bool valid = token < p.M;
+      float x[32];
 #pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2)
+      for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) x[t2][16 * db + i] = acc[2 * tp + t2][db][i] * tg.out_scale;   // x index = ks*8 + j
+        for (int j = 0; j < 8; ++j) x[ks * 8 + j] = valid ? acc[t][2 * ks + (j >> 2)][j & 3] * tg.out_scale : 0.f;
       if (bias) {
 #pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2)
+        for (int ks = 0; ks < 4; ++ks) {
+          const f32x4 b0 = *(const f32x4*)(bias + 32 * ks + 8 * g), b1 = *(const f32x4*)(bias + 32 * ks + 8 * g + 4);
 #pragma unroll
-          for (int ks = 0; ks < 8; ++ks) {
-            const f32x4 b0 = *(const f32x4*)(bias + 16 * ks + 8 * hh), b1 = *(const f32x4*)(bias + 16 * ks + 8 * hh + 4);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              x[t2][ks * 8 + j] += b0[j];
-              x[t2][ks * 8 + 4 + j] += b1[j];
-            }
+          for (int j = 0; j < 4; ++j) {
+            x[ks * 8 + j] += valid ? b0[j] : 0.f;
+            x[ks * 8 + 4 + j] += valid ? b1[j] : 0.f;
           }
+        }
       }
-      if constexpr (EPI == kEpiKImg || EPI == kEpiAImg) {
+      if constexpr (EPI == kEpiKImg) {
         const RowTransform tf{tg.norm_w, tg.norm_eps, tg.rope_mode, tg.cos_t, tg.sin_t};
-        float nmax = 0.f, amax = 0.f;
+        norm_rope_quarter(x, tf, valid ? token : 0, valid, g);
+        // kept for the tile-wide reductions below
 #pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-          const int token = tok0 + 32 * t2 + r;
-          const bool valid = token < p.M;
-          if (!valid) {
+        for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int i = 0; i < 64; ++i) x[t2][i] = 0.f;
-          }
-          norm_rope_row(x[t2], tf, valid ? token : 0, valid, hh);
-          float ssq = 0.f;
+          for (int j = 0; j < 8; ++j) acc[t][2 * ks + (j >> 2)][j & 3] = x[ks * 8 + j];
+      } else if constexpr (EPI == kEpiAImg) {
+        // operand images of these GEMMs: [16-token block][k-step], this lane's piece ks at its own place in image ks
+        char* rec = tg.out + (int64_t)(m_tile * 16 + tq * 4 + t) * tg.out_blk_stride;
 #pragma unroll
-          for (int i = 0; i < 64; ++i) {
-            ssq += x[t2][i] * x[t2][i];
-            amax = fmaxf(amax, fabsf(x[t2][i]));
-          }
-          nmax = fmaxf(nmax, ssq + xhalf(ssq));
-        }
-        if (tg.norm_max) {
-          nmax = sqrtf(wave_max(nmax));
-          if (lane == 0) atomicMax(tg.norm_max + head, __float_as_uint(nmax));
-        }
-        char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
-        if (!tg.fp8) {
+        for (int ks = 0; ks < 4; ++ks) {
+          bf16x8 v;
 #pragma unroll
-          for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-              bf16x8 t;
-#pragma unroll
-              for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[t2][ks * 8 + j];
-              // kEpiKImg: the attention kernel's K tile; kEpiAImg: operand images of these GEMMs ([token block][k-step])
-              if constexpr (EPI == kEpiKImg) *(bf16x8*)(rec + k_piece_offset(32 * t2 + r, 2 * ks + hh)) = t;
-              else *(bf16x8*)(rec + t2 * tg.out_sub_stride + (ks * 64 + lane) * 16) = t;
-            }
-        } else {
-          amax = wave_max(amax);
-          const float scale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
-          const float inv = 1.0f / scale;
-          if (lane == 0) tg.scale_out[(int64_t)head * tg.scale_head_stride + tile] = scale;
-#pragma unroll
-          for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-            for (int c2 = 0; c2 < 2; ++c2) {
-              const i32x4 q0 = quant_fp8_chunk(x[t2], 2 * c2, inv), q1 = quant_fp8_chunk(x[t2], 2 * c2 + 1, inv);
-#pragma unroll
-              for (int a = 0; a < 2; ++a) {
-                const i32x4 t = {q0[2 * a], q0[2 * a + 1], q1[2 * a], q1[2 * a + 1]};
-                *(i32x4*)(rec + k8_chunk_offset(32 * t2 + r, 2 * (4 * c2 + a) + hh)) = t;
-              }
-            }
+          for (int j = 0; j < 8; ++j) v[j] = (__bf16)x[ks * 8 + j];
+          *(bf16x8*)(rec + (ks * 64 + lane) * 16) = v;
         }
       } else {
         // row-major bf16 rows: y = residual + gate[row_index] * (acc*scale + bias); 16-byte pieces per lane
+        if (!valid) continue;
+        __bf16* orow = (__bf16*)tg.out + (int64_t)token * tg.out_row_stride + (int64_t)head * tg.out_head_elems;
+        const __bf16* res = tg.residual ? (const __bf16*)tg.residual + (int64_t)token * tg.res_row_stride + head * 128 : nullptr;
+        const __bf16* gate = tg.gate ? (const __bf16*)tg.gate + (int64_t)(tg.row_index ? tg.row_index[token] : 0) * tg.gate_row_stride + head * 128
+                                     : nullptr;
 #pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-          const int token = tok0 + 32 * t2 + r;
-          if (token >= p.M) continue;
-          __bf16* orow = (__bf16*)tg.out + (int64_t)token * tg.out_row_stride + (int64_t)head * tg.out_head_elems;
-          const __bf16* res = tg.residual ? (const __bf16*)tg.residual + (int64_t)token * tg.res_row_stride + head * 128 : nullptr;
-          const __bf16* gate = tg.gate ? (const __bf16*)tg.gate + (int64_t)(tg.row_index ? tg.row_index[token] : 0) * tg.gate_row_stride + head * 128
-                                       : nullptr;
+        for (int ks = 0; ks < 4; ++ks) {
+          const int d0 = 32 * ks + 8 * g;
+          bf16x8 o, gv, rv;
+          if (gate) gv = *(const bf16x8*)(gate + d0);
+          if (res) rv = *(const bf16x8*)(res + d0);
 #pragma unroll
-          for (int ks = 0; ks < 8; ++ks) {
-            const int d0 = 16 * ks + 8 * hh;
-            bf16x8 o;
-            bf16x8 gv, rv;
-            if (gate) gv = *(const bf16x8*)(gate + d0);
-            if (res) rv = *(const bf16x8*)(res + d0);
+          for (int j = 0; j < 8; ++j) {
+            float v = x[ks * 8 + j];
+            if (gate) v *= (float)gv[j];
+            if (res) v += (float)rv[j];
+            o[j] = (__bf16)v;
+          }
+          *(bf16x8*)(orow + d0) = o;
+        }
+      }
+    }
+    if constexpr (EPI == kEpiKImg) {
+      // the wave's 64 tokens are one K tile: largest row norm, fp8 scale, then every piece at its place in the tile
+      float nmax = 0.f, amax = 0.f;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        float ssq = 0.f;
+#pragma unroll
+        for (int fb = 0; fb < 8; ++fb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            ssq += acc[t][fb][i] * acc[t][fb][i];
+            amax = fmaxf(amax, fabsf(acc[t][fb][i]));
+          }
+        nmax = fmaxf(nmax, wave_sum_groups(ssq));
+      }
+      if (tg.norm_max) {
+        nmax = sqrtf(wave_max(nmax));
+        if (lane == 0) atomicMax(tg.norm_max + head, __float_as_uint(nmax));
+      }
+      char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
+      if (!tg.fp8) {
+        // K tile image (half, ks, kb2) of 16-token block t = 2*half + kb2: this lane's piece ks at its own place
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) {
+            bf16x8 v;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = (__bf16)acc[t][2 * ks + (j >> 2)][j & 3];
+            *(bf16x8*)(rec + ((((t >> 1) * 4 + ks) * 2 + (t & 1)) * 64 + lane) * 16) = v;
+          }
+      } else {
+        amax = wave_max(amax);
+        const float scale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
+        const float inv = 1.0f / scale;
+        if (lane == 0) tg.scale_out[(int64_t)head * tg.scale_head_stride + tile] = scale;
+        // fp8 K tile: key block t is 2 KiB, chunk c2 of a lane holds its pieces ks = 2*c2 and 2*c2 + 1
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int c2 = 0; c2 < 2; ++c2) {
+            float lo[8], hi[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-              float v = x[t2][ks * 8 + j];
-              if (gate) v *= (float)gv[j];
-              if (res) v += (float)rv[j];
-              o[j] = (__bf16)v;
+              lo[j] = acc[t][4 * c2 + (j >> 2)][j & 3];
+              hi[j] = acc[t][4 * c2 + 2 + (j >> 2)][j & 3];
             }
-            *(bf16x8*)(orow + d0) = o;
+            const i32x2 q0 = quant_fp8_piece(lo, inv), q1 = quant_fp8_piece(hi, inv);
+            *(i32x4*)(rec + ((t * 2 + c2) * 64 + lane) * 16) = i32x4{q0[0], q0[1], q1[0], q1[1]};
           }
-        }
       }
     }
   }
@@ -352,10 +422,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void gemm_kernel(GemmParams p) {
   while (t + 1 < p.n_targets && n_tile >= p.tg[t].n_tiles) { n_tile -= p.tg[t].n_tiles; ++t; }
   const GemmTarget& tg = p.tg[t];
   switch (tg.epi) {
-    case kEpiRows: gemm_tile<kEpiRows, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
-    case kEpiKImg: gemm_tile<kEpiKImg, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
-    case kEpiAImg: gemm_tile<kEpiAImg, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
-    default: gemm_tile<kEpiVImg, WAVES>(p, tg, m_tile, n_tile, lds_raw); break;
+    case kEpiRows: gemm_tile<kEpiRows>(p, tg, m_tile, n_tile, lds_raw); break;
+    case kEpiKImg: gemm_tile<kEpiKImg>(p, tg, m_tile, n_tile, lds_raw); break;
+    case kEpiAImg: gemm_tile<kEpiAImg>(p, tg, m_tile, n_tile, lds_raw); break;
+    default: gemm_tile<kEpiVImg>(p, tg, m_tile, n_tile, lds_raw); break;
   }
 }
 
@@ -369,10 +439,11 @@ hipError_t launch_gemm(const GemmParams& p, hipStream_t st) {
 // Rows -> operand images, optionally through the AdaLN modulation of the block:
 //   y = norm(x) * (1 + scale[row_index]) + shift[row_index]
 // with norm = LayerNorm without affine parameters, RMSNorm without weight, or nothing, statistics in fp32.
-// One wave per row: lane l holds the 16-byte pieces l, l + 64, ... of the row.  Image of (32-row block rb,
-// k-step ks) at ((rb * K/16 + ks) * 64 + lane') * 16 with lane' = 32 * ((k / 8) & 1) + row % 32.
+// One wave per row: lane l holds the 16-byte pieces l, l + 64, ... of the row.  Piece pc (elements 8*pc .. +7) of row r
+// belongs to image (16-row block r/16, k-step pc/4), lane 16*(pc%4) + r%16: byte ((r/16)*(K/32) + pc/4)*1024 +
+// (16*(pc%4) + r%16)*16.
 // `head_perm`: the rows are weight rows (output features) and are stored permuted inside each 128-row head
-// (see gemm_tile): image row 32*db + 8*a + 4*hh + b takes source row 32*db + 16*(a>>1) + 8*hh + 4*(a&1) + b.
+// (see gemm_tile): image row 16*fb + 4*g + i takes source row 32*(fb/2) + 8*g + 4*(fb%2) + i.
 constexpr int kPackMaxPieces = 8;  // 16-byte pieces per lane: rows of up to 64 * 8 * 8 = 4096 elements
 
 template <int NORM>
@@ -382,8 +453,8 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackParams p) {
   if (row >= p.rows_padded) return;
   int src = row;
   if (p.head_perm) {
-    const int in_head = row & 127, db = in_head >> 5, q = in_head & 31, a = q >> 3, h2 = (q >> 2) & 1, b = q & 3;
-    src = (row & ~127) + 32 * db + 16 * (a >> 1) + 8 * h2 + 4 * (a & 1) + b;
+    const int in_head = row & 127, fb = in_head >> 4, g = (in_head >> 2) & 3, i = in_head & 3;
+    src = (row & ~127) + 32 * (fb >> 1) + 8 * g + 4 * (fb & 1) + i;
   }
   const bool valid = src < p.rows;
   const int pieces = p.K / 8;                        // 16-byte pieces per row
@@ -430,7 +501,7 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackParams p) {
       }
     }
   }
-  char* ob = p.out + (int64_t)(row >> 5) * p.out_blk_stride;
+  char* ob = p.out + (int64_t)(row >> 4) * p.out_blk_stride;
 #pragma unroll
   for (int c = 0; c < kPackMaxPieces; ++c) {
     const int pc = lane + 64 * c;
@@ -438,7 +509,7 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackParams p) {
     bf16x8 t;
 #pragma unroll
     for (int j = 0; j < 8; ++j) t[j] = (__bf16)v[c][j];
-    *(bf16x8*)(ob + ((int64_t)(pc >> 1) * 64 + 32 * (pc & 1) + (row & 31)) * 16) = t;
+    *(bf16x8*)(ob + ((int64_t)(pc >> 2) * 64 + 16 * (pc & 3) + (row & 15)) * 16) = t;
   }
 }
 

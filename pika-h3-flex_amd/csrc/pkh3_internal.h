@@ -68,8 +68,8 @@ struct FwdParams {
   const int* row_cnt;       // [B] valid keys after compaction, or null (= Sk)
   void* o;
   int64_t o_sb, o_ss, o_sh;
-  int o_images;             // write O as 32-row operand images [row block][H*8 k-steps] instead of [B, Sq, H, D] rows
-  int64_t o_img_blk_stride; // bytes between consecutive 32-row blocks of those images
+  int o_images;             // write O as 16-row operand images [row block][H*4 k-steps] instead of [B, Sq, H, D] rows
+  int64_t o_img_blk_stride; // bytes between consecutive 16-row blocks of those images
   int B, H, Sq, Sk;
   int nQ64, nKt;
   float c;                  // softmax_scale * log2(e)
@@ -95,7 +95,7 @@ struct GemmTarget {
   int n;                   // features of this target (multiple of 128)
   int n_tiles;             // 256-feature workgroup tiles: ceil(n / 256)
   const char* w_img;       // packed weights [feature block][k-step], head-permuted rows unless epi == kEpiVImg
-  int64_t w_blk_stride;    // bytes between consecutive 32-feature blocks
+  int64_t w_blk_stride;    // bytes between consecutive 16-feature blocks
   const float* bias;       // [n] fp32 in original feature order, or null
   float out_scale;         // accumulator * out_scale (+ bias)
   // second K segment (LoRA): activations from the down-projected rows of this target, weights from B
@@ -107,8 +107,7 @@ struct GemmTarget {
   // output
   char* out;
   int64_t out_head_stride; // image epilogues: bytes between heads
-  int64_t out_blk_stride;  // image epilogues: bytes between 64-token tiles
-  int out_sub_stride;      // kEpiAImg: bytes between the two 32-token blocks of a 64-token pair
+  int64_t out_blk_stride;  // kEpiKImg / kEpiVImg: bytes between 64-token tiles; kEpiAImg: between 16-token blocks
   int64_t out_row_stride;  // kEpiRows: elements between token rows
   int out_head_elems;      // kEpiRows: elements between heads
   // kEpiKImg
@@ -131,7 +130,7 @@ struct GemmTarget {
 
 struct GemmParams {
   const char* a_img;       // activations [token block][k-step]
-  int64_t a_blk_stride;    // bytes between consecutive 32-token blocks
+  int64_t a_blk_stride;    // bytes between consecutive 16-token blocks
   int nk1;                 // 32-wide k-chunks of the first segment
   int M;                   // tokens
   int m_tiles, n_tiles;    // 256 x 256 workgroup tiles
@@ -143,7 +142,7 @@ struct GemmParams {
 struct PackParams {
   const void* x;           // bf16 [rows, row_stride]
   int64_t row_stride;      // elements
-  int rows, rows_padded;   // rows that exist / image rows to write (multiple of 32; the rest is zero)
+  int rows, rows_padded;   // rows that exist / image rows to write (multiple of 16; the rest is zero)
   int K;                   // elements per row (multiple of 16, <= 4096)
   int head_perm;
   int norm;                // kNorm*
@@ -153,7 +152,7 @@ struct PackParams {
   int64_t table_stride;
   const int* row_index;    // [rows] table row of each row, or null (row 0)
   char* out;
-  int64_t out_blk_stride;  // bytes between consecutive 32-row blocks
+  int64_t out_blk_stride;  // bytes between consecutive 16-row blocks
 };
 
 hipError_t launch_gemm(const GemmParams& p, hipStream_t st);

@@ -17,17 +17,16 @@ def _r(*shape, seed=0, std=1.0):
 
 
 def _unpack(buf, rows, K):
-    """Operand images -> matrix: image (rb, ks) holds rows 32*rb..+31; lane 32*hh + r carries elements
-    16*ks + 8*hh + 0..7 of row 32*rb + r."""
-    img = buf.view(torch.bfloat16).view(-1, K // 16, 2, 32, 8)      # [rb, ks, hh, r, j]
+    """Operand images -> matrix: image (rb, ks) holds rows 16*rb..+15; lane 16*g + c carries elements
+    32*ks + 8*g + 0..7 of row 16*rb + c."""
+    img = buf.view(torch.bfloat16).view(-1, K // 32, 4, 16, 8)      # [rb, ks, g, c, j]
     return img.permute(0, 3, 1, 2, 4).reshape(-1, K)[:rows]
 
 
 def _head_perm_source(rho):
-    """Source row (inside its 128-row head) of image row ``rho``: 32*db + 8*a + 4*h + b <- 32*db + 16*(a>>1) + 8*h + 4*(a&1) + b."""
-    db, q = rho // 32, rho % 32
-    a, h, b = q // 8, (q // 4) % 2, q % 4
-    return 32 * db + 16 * (a >> 1) + 8 * h + 4 * (a & 1) + b
+    """Source row (inside its 128-row head) of image row ``rho``: 16*fb + 4*g + i <- 32*(fb//2) + 8*g + 4*(fb%2) + i."""
+    fb, g, i = rho // 16, (rho // 4) % 4, rho % 4
+    return 32 * (fb // 2) + 8 * g + 4 * (fb % 2) + i
 
 
 def test_pack_layout_matches_its_index_formula():
@@ -402,7 +401,7 @@ def test_attention_writes_the_out_projection_images(S, H, variant):
     got = pk.attention(q, k, v, out=img, out_images=True, **opts)
     torch.cuda.synchronize()
     assert got is img
-    live = ((S + 31) // 32) * (H * 128 // 16) * 1024            # bytes of the 32-row blocks that hold rows
+    live = ((S + 31) // 32) * 2 * (H * 128 // 32) * 1024        # bytes of the 32-row blocks that hold rows
     assert torch.equal(img[:live], want[:live])
     assert bool((img[live:] == 0xAB).all())                     # blocks past the last row are left alone
     with pytest.raises(ValueError):
