@@ -35,7 +35,7 @@ MEASURED_TRAFFIC = {
     "joint": (4.51e9, "profiles/attn_fwd_kernel_joint_bf16.md"),
     "cross": (6.15e8, "profiles/attn_fwd_kernel_cross_short_key.md"),
 }
-GEMM_TRAFFIC = (6.28e9, "profiles/gemm_kernel_480p_block.md")  # to_q/to_k/to_v launch of the 480p block
+GEMM_TRAFFIC = (7.54e9, "profiles/gemm_kernel_480p_block.md")  # to_q/to_k/to_v launch of the 480p block
 
 
 def host_cpu():
