@@ -575,11 +575,13 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
     __syncthreads();                                                                                    \
     const char* kbuf = lds[slot];                                                                       \
+    const int tile = entry(i);                                                                          \
+    qk_tile<FP8, LEAN, (MASKED) ? 2 : 4>(w, kbuf, kbuf + kKBytes, lane);                                \
+    /* the copies of the tile two ahead are issued under the MFMAs of S^T, not in front of them: right */ \
+    /* after the barrier their scalar address chain would run in every wave at once with the pipe idle */ \
     if (i + kAhead < nt) dma(entry(i + kAhead), slot_prev);                                             \
     slot_prev = slot;                                                                                   \
     slot = slot == kRingT - 1 ? 0 : slot + 1;                                                           \
-    const int tile = entry(i);                                                                          \
-    qk_tile<FP8, LEAN, (MASKED) ? 2 : 4>(w, kbuf, kbuf + kKBytes, lane);                                \
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
     softmax_pv_tile<FP8, STATIC, LEAN, MASKED>(w, kbuf + kKBytes, ct, tail, lane);                      \
   }
@@ -591,12 +593,14 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
     __syncthreads();                                                                                    \
     const char* hbuf = ring + slot * kHalfBytes;                                                        \
+    const int half = h_begin + i;                                                                       \
+    const bool live = FULL || i < n_mine;                                                               \
+    if (live) qk_half<FP8, true>(w, hbuf, hbuf + kKHalfB, lane);                                        \
+    /* copies of the half two ahead: under the MFMAs of S^T (see the whole-tile loop) */               \
     if (i + 2 < n_mine) dma_short(h_begin + i + 2, slot_prev);                                          \
     slot_prev = slot;                                                                                   \
     slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
-    const int half = h_begin + i;                                                                       \
-    if (FULL || i < n_mine) {                                                                           \
-      qk_half<FP8, true>(w, hbuf, hbuf + kKHalfB, lane);                                                \
+    if (live) {                                                                                         \
       const float ct = FP8 ? c * uniform_load(kscale, half >> 1) : c;                                   \
       softmax_pv_half<FP8, STATIC, true, FULL>(w, ct, sk - 32 * half, lane, hbuf + kKHalfB);            \
     }                                                                                                   \
@@ -705,14 +709,16 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   for (int it = 0; it < n_iter; ++it) {                                                                 \
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
     __syncthreads();                                                                                    \
-    if (it + kStages2 - 1 < 2 * n_mine) dma_half(it + kStages2 - 1, st2_free);                          \
     const char* hbuf = lds_raw + (st2 * kSparseRows + r) * kHalfBytes;                                  \
+    const int st2_write = st2_free;                                                                     \
     st2_free = st2;                                                                                     \
     st2 = st2 == kStages2 - 1 ? 0 : st2 + 1;                                                            \
-    if (it >= 2 * n_mine) continue; /* wave-uniform: this row-block has run out of tiles */             \
+    if (it >= 2 * n_mine) continue; /* wave-uniform: this row-block has run out of tiles (and of copies) */ \
     const int tile = uniform_load(mine, it >> 1);                                                       \
     /* the running-max copy needs registers for the rescale: it takes the lean read-ahead (4 images) */ \
     qk_half<FP8, !STATIC>(w, hbuf, hbuf + kKHalf, lane);                                                \
+    /* copies of the next half tile of this row-block: under the MFMAs of S^T (see the whole-tile loop) */ \
+    if (it + kStages2 - 1 < 2 * n_mine) dma_half(it + kStages2 - 1, st2_write);                         \
     const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
     const int lim = (tail && tile == nkt - 1) ? tail - 32 * (it & 1) : 32;                              \
     softmax_pv_half<FP8, STATIC, !STATIC>(w, ct, lim, lane, hbuf + kKHalf);                             \
