@@ -415,6 +415,7 @@ int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream)
   if (p->S != a->Sq) return fail(PKH3_ESHAPE, "qkv_proj: S = %d but the attention call has Sq = %d", p->S, a->Sq);
   if (p->K < 32 || (p->K % 32) || p->K > 4096) return fail(PKH3_ESHAPE, "qkv_proj: K must be a multiple of 32 in [32, 4096], got %d", p->K);
   if (!p->x_img || misaligned16(p->x_img)) return fail(PKH3_ENULL, "qkv_proj: x_img is NULL or misaligned");
+  if (a->q_sh > INT32_MAX) return fail(PKH3_ESTRIDE, "qkv_proj: q head stride too large");
   const pkh3_linear* lin[3] = {&p->q, &p->k, &p->v};
   const char* names[3] = {"q", "k", "v"};
   bool any_lora = false;
@@ -485,7 +486,6 @@ int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream)
     GemmTarget& v = g.tg[2];
     v.epi = kEpiVImg; v.out = L.vp.out; v.out_head_stride = L.vp.out_bh_stride; v.out_blk_stride = L.vp.out_tile_stride;
   }
-  if (a->q_sh > INT32_MAX) return fail(PKH3_ESTRIDE, "qkv_proj: q head stride too large");
   if ((e = launch_gemm(g, st)) != hipSuccess) return hip_fail(e, "qkv projection");
   g_err[0] = 0;
   return PKH3_OK;

@@ -229,7 +229,8 @@ class PikaH3AttnProcessor:
         if rope_cos_sin is not None:
             opts.update(rope_mode=self.rope_mode, rope_q=rope_cos_sin, rope_k=rope_cos_sin)
         # the attention kernel writes its output as the operand images of the out-projection: no packing pass
-        o_img = qkv_attention(x_img, S, packed["q"], packed["k"], packed["v"], heads=H, out_images=True, **opts)
+        o_img = qkv_attention(x_img, S, packed["q"], packed["k"], packed["v"], heads=H, out_images=True,
+                              workspace=self._workspace, **opts)
         res = None
         if residual is not None:
             res = residual[0] if residual.dim() == 3 else residual

@@ -113,7 +113,9 @@ class PackedLinear:
         N, K = weight.shape
         pl = PackedLinear(pack_weight(weight, head_perm=head_perm), int(N), int(K))
         if bias is not None:
-            pl.bias = bias.detach().to(device=weight.device, dtype=torch.float32).contiguous()
+            if bias.numel() != N:
+                raise ValueError(f"bias has {bias.numel()} elements, the layer has {N} outputs")
+            pl.bias = bias.detach().to(device=weight.device, dtype=torch.float32).contiguous().view(N)
         if (lora_a is None) != (lora_b is None):
             raise ValueError("lora_a and lora_b go together")
         if lora_a is not None:
@@ -138,6 +140,12 @@ class PackedLinear:
         return PackedLinear.from_weights(base.weight.detach().to(torch.bfloat16), getattr(base, "bias", None),
                                          head_perm=head_perm, **kw)
 
+    def check_device(self, name: str, device) -> None:
+        """Every buffer of the layer is dereferenced by kernels running on ``device``."""
+        for part, t in (("w_img", self.w_img), ("bias", self.bias), ("lora_a_img", self.lora_a_img), ("lora_b_img", self.lora_b_img)):
+            if t is not None:
+                _on_device(f"{name}.{part}", t, device)
+
     def c_struct(self) -> _lib.Linear:
         s = _lib.Linear()
         s.w_img = self.w_img.data_ptr()
@@ -148,29 +156,43 @@ class PackedLinear:
         return s
 
 
+def _scratch(workspace, device, nbytes: int) -> torch.Tensor:
+    """``workspace``: None (allocate), a uint8 device tensor (used when large enough) or a callable
+    ``(device, nbytes) -> tensor``, as in :func:`ops.attention`."""
+    if callable(workspace):
+        workspace = workspace(device, nbytes)
+    if workspace is None or workspace.numel() * workspace.element_size() < nbytes:
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    _on_device("workspace", workspace, device)
+    return workspace
+
+
 def qkv_attention(x_img: torch.Tensor, S: int, q: PackedLinear, k: PackedLinear, v: PackedLinear, *, heads: int,
-                  out: Optional[torch.Tensor] = None, return_q: bool = False, **opts) -> torch.Tensor:
+                  out: Optional[torch.Tensor] = None, return_q: bool = False, workspace=None, **opts) -> torch.Tensor:
     """One self-attention call from packed activations: ``to_q / to_k / to_v`` (+ adapters) with the K side's
     norm + rotation (+ fp8 quantisation) and the K/V layout in the GEMM epilogue, then the attention kernel on
     what the GEMM left in the workspace.  ``opts`` are those of :func:`ops.fill_args` (norm weights, rope
     tables, ``fp8_qk``, ``block_mask`` ...).  Returns O ``[1, S, H, D]`` bf16 (and Q when ``return_q``); with
     ``out_images=True`` O comes back as the packed operand images :func:`out_proj` takes (``o_img=``), written
-    by the attention kernel itself."""
+    by the attention kernel itself.  ``workspace`` as in :func:`ops.attention` (the K/V images live there)."""
     lib = _lib.load()
     dev = x_img.device
+    if not x_img.is_cuda:
+        raise ValueError(f"x_img must live in device memory (got {dev}); the HIP library is the only compute path")
     K = q.K
     for name, pl in (("q", q), ("k", k), ("v", v)):
         if pl.N != heads * HEAD_DIM or pl.K != K:
             raise ValueError(f"{name} projection is [{pl.N}, {pl.K}], expected [{heads * HEAD_DIM}, {K}]")
-    if x_img.dtype != torch.uint8 or x_img.numel() < packed_bytes(S, K):
+        pl.check_device(name, dev)
+    if x_img.dtype != torch.uint8 or not x_img.is_contiguous() or x_img.numel() < packed_bytes(S, K):
         raise ValueError("x_img is not a packed [S, K] activation buffer")
     qt = torch.empty((1, S, heads, HEAD_DIM), dtype=torch.bfloat16, device=dev)
     if out is None:
         out = (torch.empty(packed_bytes(S, heads * HEAD_DIM), dtype=torch.uint8, device=dev) if opts.get("out_images")
                else torch.empty_like(qt))
     args, keep = fill_args(qt, None, None, out, kv_prepared=True, **opts)
-    ws = torch.empty(workspace_bytes(args), dtype=torch.uint8, device=dev)
-    args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+    ws = _scratch(workspace, dev, workspace_bytes(args))
+    args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
     pa = _lib.QkvArgs()
     pa.x_img, pa.S, pa.K = x_img.data_ptr(), int(S), int(K)
     pa.q, pa.k, pa.v = q.c_struct(), k.c_struct(), v.c_struct()
@@ -203,6 +225,8 @@ def out_proj(o: Optional[torch.Tensor], proj: PackedLinear, *, gate: Optional[to
         S, K = int(rows), proj.K
         if o_img.dtype != torch.uint8 or not o_img.is_contiguous() or o_img.numel() < packed_bytes(S, K):
             raise ValueError("o_img is not a packed [rows, K] activation buffer")
+        if not o_img.is_cuda:
+            raise ValueError(f"o_img must live in device memory (got {o_img.device}); the HIP library is the only compute path")
         dev = o_img.device
     else:
         o = _rows_bf16("o", o)
@@ -211,6 +235,7 @@ def out_proj(o: Optional[torch.Tensor], proj: PackedLinear, *, gate: Optional[to
             raise ValueError(f"o has {K} columns, the projection expects {proj.K}")
         dev = o.device
         o_img = pack_rows(o)
+    proj.check_device("proj", dev)
     y = torch.empty((S, proj.N), dtype=torch.bfloat16, device=dev)
     a = _lib.OutArgs()
     a.o_img, a.S, a.K, a.N = o_img.data_ptr(), S, K, proj.N

@@ -318,3 +318,22 @@ def test_projection_front_end_refuses_host_tensors():
     with pytest.raises(ValueError):
         P.packed_bytes(8, 48)
     assert P.packed_bytes(300, 64) == 512 * 64 * 2
+
+
+def test_fused_front_end_refuses_host_buffers():
+    """qkv_attention / out_proj hand raw pointers to kernels: a host buffer must be stopped on the host."""
+    import torch
+
+    from pika_h3_flex_amd import projections as P
+
+    S, K, H = 16, 128, 1
+    img = torch.zeros(P.packed_bytes(S, K), dtype=torch.uint8)
+    lin = P.PackedLinear(torch.zeros(P.packed_bytes(128, K), dtype=torch.uint8), 128, K)
+    with pytest.raises(ValueError, match="device memory"):
+        P.qkv_attention(img, S, lin, lin, lin, heads=H)
+    with pytest.raises(ValueError, match="device memory"):
+        P.out_proj(None, lin, o_img=img, rows=S)
+    with pytest.raises(ValueError, match="either o or o_img"):
+        P.out_proj(None, lin)
+    with pytest.raises(ValueError, match="number of rows"):
+        P.out_proj(None, lin, o_img=img)
