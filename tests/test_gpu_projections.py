@@ -406,3 +406,69 @@ def test_attention_writes_the_out_projection_images(S, H, variant):
     assert bool((img[live:] == 0xAB).all())                     # blocks past the last row are left alone
     with pytest.raises(ValueError):
         pk.attention(q.expand(2, -1, -1, -1), k.expand(2, -1, -1, -1), v.expand(2, -1, -1, -1), out=img, out_images=True, **opts)
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_random_projection_combinations(seed):
+    """Seeded sweep over what the fixed cases above leave out: row counts around the 16-row image and the 256-row tile
+    (1, 2, 15..17, 255..257 ...), an activation width different from heads x 128, adapters and biases on some of the
+    three targets only, both output forms of the attention call, each followed by the out-projection."""
+    import random
+
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as AO
+    from oracle import projection_oracle as PO
+    from pika_h3_flex_amd import projections as P
+
+    rng = random.Random(seed)
+    for case in range(20):
+        S = rng.choice([1, 2, 15, 16, 17, 31, 33, 47, 63, 64, 65, 255, 256, 257, 300, 511, 513, 777, 1030])
+        H, K = rng.choice([1, 2, 3]), rng.choice([32, 96, 128, 256, 384, 544])
+        C = H * D
+        variant = rng.choice(["bf16", "bf16", "fp8", "sparse", "norope", "half"])
+        base = 100000 * seed + 1000 * case
+        x = _r(S, K, seed=base + 900).to(torch.bfloat16)
+        lin = {n: _linear(C, K, base + 10 * i, lora=rng.random() < 0.6, bias=rng.random() < 0.6) for i, n in enumerate("qkv")}
+        wq, wk = 1.0 + 0.1 * _r(D, seed=50), 1.0 + 0.1 * _r(D, seed=51)
+        opts, ref_opts = dict(q_norm_weight=wq.cuda(), k_norm_weight=wk.cuda()), dict(q_norm_weight=wq, k_norm_weight=wk)
+        if variant != "norope":
+            pos = torch.rand((S, 3), generator=torch.Generator().manual_seed(base), dtype=torch.float64) * 20
+            mode = pk.ROPE_HALF if variant == "half" else pk.ROPE_INTERLEAVED
+            opts.update(rope_mode=mode, rope_q=pk.rope_tables(pos.cuda()))
+            ref_opts.update(rope_mode=mode, rope_q=AO.rope_tables(pos))
+        if variant == "fp8":
+            opts.update(fp8_qk=True)
+            ref_opts.update(fp8_qk=True)
+        if variant == "sparse":
+            n = (S + 63) // 64
+            tm = (torch.rand((n, n), generator=torch.Generator().manual_seed(base + 3)) < 0.5) | torch.eye(n, dtype=torch.bool)
+            opts.update(block_mask=pk.BlockMask.from_dense(tm, device="cuda"))
+            ref_opts.update(tile_map=tm)
+        as_images = rng.random() < 0.5
+        out, q = P.qkv_attention(P.pack_rows(x.cuda()), S, _packed(lin["q"]), _packed(lin["k"]), _packed(lin["v"], head_perm=False),
+                                 heads=H, return_q=True, out_images=as_images, **opts)
+        n_out = rng.choice([128, 256, 384])
+        lo = _linear(n_out, C, base + 500, lora=rng.random() < 0.5, bias=rng.random() < 0.5)
+        q_ref, k_ref, v_ref = (PO.lora_linear(x, **lin[n]).view(1, S, H, D) for n in "qkv")
+        r = lambda t: t.to(torch.bfloat16)
+        o_ref = AO.reference_layer(r(q_ref), r(k_ref), r(v_ref), **ref_opts)
+        if as_images:
+            y = P.out_proj(None, _packed(lo), o_img=out, rows=S)
+            y_ref = PO.lora_linear(r(o_ref).view(S, C), **lo)
+            err_o, cos_o = 0.0, 1.0  # O is checked through y
+        else:
+            y = P.out_proj(out.view(S, C), _packed(lo))
+            y_ref = PO.lora_linear(out.cpu().view(S, C), **lo)
+            err_o, cos_o = AO.max_abs_and_cosine(out.cpu(), o_ref)
+        torch.cuda.synchronize()
+        err_q, cos_q = AO.max_abs_and_cosine(q.cpu(), q_ref)
+        err_y, cos_y = AO.max_abs_and_cosine(y.cpu(), y_ref)
+        label = (f"seed {seed} case {case}: S={S} H={H} K={K} {variant} images={as_images} N_out={n_out} "
+                 f"lora={['lora_a' in lin[n] for n in 'qkv']} bias={['bias' in lin[n] for n in 'qkv']}: "
+                 f"Q {err_q:.2e}/{cos_q:.6f} O {err_o:.2e}/{cos_o:.6f} y {err_y:.2e}/{cos_y:.6f}")
+        print(label, flush=True)
+        assert torch.isfinite(y.float()).all(), label
+        fp8 = variant == "fp8"
+        assert err_q <= 2e-2 and cos_q >= 0.9999, label
+        assert cos_o >= (0.995 if fp8 else 0.9999) and (fp8 or err_o <= 2e-2), label
+        assert cos_y >= (0.995 if fp8 and as_images else 0.9999), label
