@@ -50,6 +50,9 @@ int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = tru
   if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Sk < 1) return fail(PKH3_ESHAPE, "B, H, Sq, Sk must be >= 1");
   if (a->B > 65535 || a->H > 65535) return fail(PKH3_ESHAPE, "B and H must be <= 65535");
   if (a->Sq > (1 << 24) || a->Sk > (1 << 24)) return fail(PKH3_ESHAPE, "Sq and Sk must be <= 2^24");
+  // workgroup counts and tile indices are 32-bit: at most 2^30 blocks of 32 queries per call
+  if ((int64_t)a->B * a->H * ((a->Sq + 31) / 32) > (1ll << 30))
+    return fail(PKH3_ESHAPE, "B * H * ceil(Sq / 32) must be <= 2^30");
   if (a->flags & ~(uint32_t)(PKH3_FLAG_FP8_QK | PKH3_FLAG_LONG_KEY_KERNEL | PKH3_FLAG_KV_PREPARED | PKH3_FLAG_O_IMAGES))
     return fail(PKH3_EARG, "unknown flag bits 0x%x", a->flags);
   if ((a->flags & PKH3_FLAG_KV_PREPARED) && (a->key_mask || a->B != 1 || a->Sq != a->Sk))

@@ -74,6 +74,8 @@ def test_workspace_bytes_host_only(lib):
     (lambda a: setattr(a, "q", 0), _lib.PKH3_ENULL),
     (lambda a: setattr(a, "Sq", 0), _lib.PKH3_ESHAPE),
     (lambda a: setattr(a, "H", 70000), _lib.PKH3_ESHAPE),
+    # 32-bit workgroup counts: B * H * ceil(Sq / 32) is bounded
+    (lambda a: (setattr(a, "B", 60000), setattr(a, "H", 60000), setattr(a, "Sq", 1 << 20)), _lib.PKH3_ESHAPE),
     (lambda a: setattr(a, "k", 0x10008), _lib.PKH3_EALIGN),
     (lambda a: setattr(a, "v_ss", 132), _lib.PKH3_ESTRIDE),
     (lambda a: setattr(a, "o_sh", -128), _lib.PKH3_ESTRIDE),
