@@ -472,3 +472,50 @@ def test_random_projection_combinations(seed):
         assert err_q <= 2e-2 and cos_q >= 0.9999, label
         assert cos_o >= (0.995 if fp8 else 0.9999) and (fp8 or err_o <= 2e-2), label
         assert cos_y >= (0.995 if fp8 and as_images else 0.9999), label
+
+
+def test_fused_block_replays_from_a_hip_graph():
+    """modulate -> q/k/v (+LoRA) -> attention -> to_out (+LoRA, gate, residual) captured into one HIP graph: the
+    library clears its reduction slots with a fill kernel and launches kernels only, so every replay on fresh
+    inputs, with eager work and synchronisation in between, must give the bits of the eager calls."""
+    import pika_h3_flex_amd as pk
+    from pika_h3_flex_amd import projections as P
+
+    S, H = 700, 2
+    C = H * D
+    dev = "cuda"
+    lin = {n: _packed(_linear(C, C, 300 + 10 * i), head_perm=(n != "v")) for i, n in enumerate("qkv")}
+    lo = _packed(_linear(C, C, 340))
+    T = 3
+    shift, scale = (_r(T, C, seed=350 + i, std=0.3).to(torch.bfloat16).to(dev) for i in range(2))
+    gate = _r(T, C, seed=352, std=0.5).to(torch.bfloat16).to(dev)
+    idx = torch.randint(0, T, (S,), generator=torch.Generator().manual_seed(353)).to(torch.int32).to(dev)
+    w = torch.ones(D, device=dev)
+    pos = torch.rand((S, 3), generator=torch.Generator().manual_seed(354), dtype=torch.float64) * 20
+    opts = dict(q_norm_weight=w, k_norm_weight=w, rope_mode=pk.ROPE_INTERLEAVED, rope_q=pk.rope_tables(pos.to(dev)))
+
+    def block(x):
+        x_img = P.adaln_modulate(x, shift=shift, scale=scale, row_index=idx)
+        o_img = P.qkv_attention(x_img, S, lin["q"], lin["k"], lin["v"], heads=H, out_images=True, **opts)
+        return P.out_proj(None, lo, gate=gate, row_index=idx, residual=x, o_img=o_img, rows=S)
+
+    x_buf = _r(S, C, seed=360).to(torch.bfloat16).to(dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        block(x_buf)  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_buf = block(x_buf)
+    for rep in range(4):
+        fresh = _r(S, C, seed=370 + rep).to(torch.bfloat16).to(dev)
+        eager = block(fresh).clone()
+        torch.cuda.synchronize()
+        x_buf.copy_(fresh)
+        y_buf.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.isfinite(y_buf.float()).all()
+        assert torch.equal(y_buf, eager), f"replay {rep} differs from the eager calls"
