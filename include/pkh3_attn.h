@@ -15,6 +15,7 @@
  *     pkh3_attn_fwd            the per-block attention between `to_v` and `to_out.0`:
  *                              QK-RMSNorm -> 3-axis RoPE from position_ids
  *                              (src/pika_h3/core/packing.py:126-135) -> softmax(QK^T * scale) V
+ *     pkh3_kv_prepare          the K/V side of that call alone, for keys and values several calls share
  *     pkh3_workspace_bytes     sizing of the scratch the call needs (caller-owned, e.g. torch.empty)
  *     pkh3_rope_tables         cos/sin tables from the [S,3] float64 position grid the layout
  *                              builder returns (src/pika_h3/core/packing.py:199, :128)
@@ -39,7 +40,7 @@
 extern "C" {
 #endif
 
-#define PKH3_VERSION 104
+#define PKH3_VERSION 105
 
 enum {
   PKH3_OK = 0,
@@ -66,8 +67,10 @@ enum {
   PKH3_FLAG_FP8_QK = 1u << 0, /* quantise normed+roped Q and K to fp8 e4m3 (OCP) with one absmax scale
                                  per (batch, head, 64-row block); P.V stays bf16 with fp32 accumulation */
   PKH3_FLAG_KV_PREPARED = 1u << 2, /* K and V already lie in `workspace` as the attention kernel reads them, written
-                                 there by pkh3_qkv_proj on the same stream with the same shapes and options: the
-                                 call skips its own K/V pass; `k` and `v` are not read and may be NULL */
+                                 there by pkh3_qkv_proj or pkh3_kv_prepare with the same B, H, Sk and K-side options:
+                                 the call skips its own K/V pass (key-mask compaction included; `key_mask` must still
+                                 be non-NULL when the keys were prepared with one); `k` and `v` are not read and may
+                                 be NULL */
   PKH3_FLAG_O_IMAGES = 1u << 3, /* `o` is not a [B, Sq, H, D] tensor but the operand-image buffer pkh3_out_proj reads
                                  (what pkh3_pack_rows would make of the [Sq, H*D] output: pkh3_packed_bytes(Sq, H*D)
                                  bytes, 16-byte aligned): the kernel's epilogue writes the images itself and the
@@ -123,6 +126,16 @@ size_t pkh3_workspace_bytes(const pkh3_attn_args* a);
 /* One attention call: the arithmetic of the DiT block's attention between the q/k/v projections and
    the output projection (module at src/pika_h3/core/loader.py:9; call site src/pika_h3/core/wrapper.py:248). */
 int pkh3_attn_fwd(const pkh3_attn_args* a, void* stream);
+
+/* The K/V side of pkh3_attn_fwd on its own: key-mask compaction, K through QK-RMSNorm, rotation and (with
+   PKH3_FLAG_FP8_QK) quantisation, K and V into `a->workspace` in the layout the attention kernel reads.  The
+   attention calls that follow pass the same B, H, Sk, K-side options (k_norm_w, norm_eps, rope_mode, k tables,
+   key_mask, PKH3_FLAG_FP8_QK) and workspace with PKH3_FLAG_KV_PREPARED added, and any q, o, Sq and block map:
+   keys and values that several calls share are prepared once -- the text keys of a block's cross-attention do not
+   change over the denoising steps of a clip (src/pika_h3/pipeline.py:13 runs the model six times on one prompt).
+   `q` and `o` of `a` are not looked at.  The K/V side occupies the head of the workspace and its size does not
+   depend on Sq or the block map; the later calls still need pkh3_workspace_bytes() of their own arguments. */
+int pkh3_kv_prepare(const pkh3_attn_args* a, void* stream);
 
 /* The same call for callers that cannot allocate device memory or pass a workspace (code under HIP graph
    capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.

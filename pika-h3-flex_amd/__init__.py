@@ -12,11 +12,11 @@ from .layout import (
 )
 from . import packing
 from . import projections
-from .ops import BlockMask, attention, rope_tables, time_attention_kernel
+from .ops import BlockMask, PreparedKV, attention, attention_prepared, prepare_kv, rope_tables, time_attention_kernel
 from .processor import PikaH3AttnProcessor
 
 __all__ = [
     "BlockMask", "PikaH3AttnProcessor", "Pkh3Error", "ROPE_HALF", "ROPE_INTERLEAVED", "ROPE_NONE",
-    "attention", "audio_position_ids", "local_window_tile_map", "packing", "projections", "rope_tables", "time_attention_kernel",
+    "PreparedKV", "attention", "attention_prepared", "audio_position_ids", "local_window_tile_map", "packing", "prepare_kv", "projections", "rope_tables", "time_attention_kernel",
     "video_position_ids",
 ]

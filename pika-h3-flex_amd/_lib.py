@@ -34,6 +34,7 @@ NOALLOC_SCRATCH_BYTES = 64 << 20  # PKH3_NOALLOC_SCRATCH_BYTES
 EXPORTS = (
     "pkh3_workspace_bytes",
     "pkh3_attn_fwd",
+    "pkh3_kv_prepare",
     "pkh3_attn_fwd_noalloc",
     "pkh3_rope_tables",
     "pkh3_version",
@@ -130,6 +131,8 @@ def load() -> C.CDLL:
     lib.pkh3_workspace_bytes.restype = C.c_size_t
     lib.pkh3_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
     lib.pkh3_attn_fwd.restype = C.c_int
+    lib.pkh3_kv_prepare.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
+    lib.pkh3_kv_prepare.restype = C.c_int
     lib.pkh3_attn_fwd_noalloc.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
     lib.pkh3_attn_fwd_noalloc.restype = C.c_int
     lib.pkh3_attn_time_kernel.argtypes = [C.POINTER(AttnArgs), C.c_void_p, C.c_int, C.POINTER(C.c_float)]

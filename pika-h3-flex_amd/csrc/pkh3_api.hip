@@ -44,7 +44,7 @@ int check_tensor(const char* name, const void* ptr, int64_t sb, int64_t ss, int6
 
 // Validation shared by pkh3_workspace_bytes (shapes/options only), pkh3_attn_fwd (everything) and
 // pkh3_attn_fwd_noalloc (everything but the caller's workspace, which it does not use).
-int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = true, bool need_kv = true) {
+int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = true, bool need_kv = true, bool need_qo = true) {
   if (!a) return fail(PKH3_ENULL, "args is NULL");
   if (a->D != kD) return fail(PKH3_EHEADDIM, "head dim must be 128, got %d", a->D);
   if (a->B < 1 || a->H < 1 || a->Sq < 1 || a->Sk < 1) return fail(PKH3_ESHAPE, "B, H, Sq, Sk must be >= 1");
@@ -55,8 +55,6 @@ int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = tru
     return fail(PKH3_ESHAPE, "B * H * ceil(Sq / 32) must be <= 2^30");
   if (a->flags & ~(uint32_t)(PKH3_FLAG_FP8_QK | PKH3_FLAG_LONG_KEY_KERNEL | PKH3_FLAG_KV_PREPARED | PKH3_FLAG_O_IMAGES))
     return fail(PKH3_EARG, "unknown flag bits 0x%x", a->flags);
-  if ((a->flags & PKH3_FLAG_KV_PREPARED) && (a->key_mask || a->B != 1 || a->Sq != a->Sk))
-    return fail(PKH3_EUNSUPPORTED, "prepared K/V (pkh3_qkv_proj) means one self-attention document: B = 1, Sq = Sk, no key mask");
   if ((a->flags & PKH3_FLAG_O_IMAGES) && a->B != 1)
     return fail(PKH3_EUNSUPPORTED, "output as operand images (PKH3_FLAG_O_IMAGES) means one document: B = 1");
   if (a->rope_mode < PKH3_ROPE_NONE || a->rope_mode > PKH3_ROPE_HALF) return fail(PKH3_EARG, "bad rope_mode %d", a->rope_mode);
@@ -68,13 +66,15 @@ int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = tru
   if ((a->flags & PKH3_FLAG_FP8_QK) && a->key_mask)
     return fail(PKH3_EUNSUPPORTED, "fp8 QK^T together with a key mask is not supported");
   if (!pointers) return PKH3_OK;
-  int rc;
-  if ((rc = check_tensor("q", a->q, a->q_sb, a->q_ss, a->q_sh, a->B, a->H))) return rc;
+  int rc = PKH3_OK;
+  if (need_qo && (rc = check_tensor("q", a->q, a->q_sb, a->q_ss, a->q_sh, a->B, a->H))) return rc;
   if (need_kv && !(a->flags & PKH3_FLAG_KV_PREPARED)) {
     if ((rc = check_tensor("k", a->k, a->k_sb, a->k_ss, a->k_sh, a->B, a->H))) return rc;
     if ((rc = check_tensor("v", a->v, a->v_sb, a->v_ss, a->v_sh, a->B, a->H))) return rc;
   }
-  if (a->flags & PKH3_FLAG_O_IMAGES) {
+  if (!need_qo) {
+    // the K/V side alone: q and o are not looked at
+  } else if (a->flags & PKH3_FLAG_O_IMAGES) {
     if (!a->o) return fail(PKH3_ENULL, "o is NULL");
     if (misaligned16(a->o)) return fail(PKH3_EALIGN, "o is not 16-byte aligned");
   } else if ((rc = check_tensor("o", a->o, a->o_sb, a->o_ss, a->o_sh, a->B, a->H))) {
@@ -106,9 +106,11 @@ WsPlan plan(const pkh3_attn_args* a) {
   w.kscale_off = off; if (fp8) off = align_up(off + bh * w.nKt * sizeof(float), 256);
   w.cnt_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * sizeof(int), 256);
   w.idx_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * a->Sk * sizeof(int), 256);
+  w.kmax_off = off;   off = align_up(off + bh * sizeof(float), 256);
+  // everything above is the K/V side and depends on B, H, Sk and the K-side options only (pkh3_kv_prepare);
+  // what follows depends on the queries of the call
   w.plan_off = off;   if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / kSparseRows) * kSparseLists * w.nKt * sizeof(int), 256);
   w.plan_cnt_off = off; if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / kSparseRows) * kSparseLists * sizeof(int), 256);
-  w.kmax_off = off;   off = align_up(off + bh * sizeof(float), 256);
   w.total = off;
   return w;
 }
@@ -176,22 +178,29 @@ int hip_fail(hipError_t e, const char* what) {
   return fail(PKH3_EHIP, "%s: %s", what, hipGetErrorString(e));
 }
 
-int run_prologue(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
+// The K/V side of a call: key-mask compaction, then V and K into the workspace in the attention kernel's layout.
+int run_kv_side(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
   hipError_t e;
   if (a->key_mask) {
     if ((e = launch_mask_compact(a->key_mask, a->B, a->Sk, L.idx, L.cnt, st)) != hipSuccess) return hip_fail(e, "mask_compact");
   }
+  // V first: it also clears the per-head slots the K pass max-reduces its row norms into
+  if ((e = launch_v_prologue(L.vp, st)) != hipSuccess) return hip_fail(e, "v prologue");
+  if ((e = launch_qk_prologue(L.kp, st)) != hipSuccess) return hip_fail(e, "k prologue");
+  return PKH3_OK;
+}
+
+int run_prologue(const pkh3_attn_args* a, const Launch& L, hipStream_t st) {
+  hipError_t e;
   if (a->blk_row_ptr) {
     char* ws = L.ws;
     if ((e = launch_sparse_plan(a->blk_row_ptr, a->blk_col_idx, (a->Sq + 63) / 64, L.w.nQ64, L.w.nKt, (int*)(ws + L.w.plan_off),
                                 kSparseLists * L.w.nKt, (int*)(ws + L.w.plan_cnt_off), st)) != hipSuccess)
       return hip_fail(e, "sparse plan");
   }
-  if (a->flags & PKH3_FLAG_KV_PREPARED) return PKH3_OK;  // pkh3_qkv_proj wrote K, V, the scales and the row-norm maxima
-  // V first: it also clears the per-head slots the K pass max-reduces its row norms into
-  if ((e = launch_v_prologue(L.vp, st)) != hipSuccess) return hip_fail(e, "v prologue");
-  if ((e = launch_qk_prologue(L.kp, st)) != hipSuccess) return hip_fail(e, "k prologue");
-  return PKH3_OK;
+  // prepared: pkh3_qkv_proj or pkh3_kv_prepare wrote K, V, the scales, the row-norm maxima and the compacted key list
+  if (a->flags & PKH3_FLAG_KV_PREPARED) return PKH3_OK;
+  return run_kv_side(a, L, st);
 }
 
 // ---- helpers of the projection entry points
@@ -296,6 +305,19 @@ int pkh3_attn_fwd(const pkh3_attn_args* a, void* stream) {
   if ((rc = run_prologue(a, L, st))) return rc;
   hipError_t e = launch_attn_fwd(L.f, st);
   if (e != hipSuccess) return hip_fail(e, "attn_fwd");
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
+int pkh3_kv_prepare(const pkh3_attn_args* a, void* stream) {
+  int rc = validate(a, true, true, /*need_kv=*/true, /*need_qo=*/false);
+  if (rc) return rc;
+  if (a->flags & PKH3_FLAG_KV_PREPARED) return fail(PKH3_EARG, "kv_prepare: PKH3_FLAG_KV_PREPARED belongs to the calls that follow");
+  Launch L;
+  build(a, a->workspace, L);
+  if (a->workspace_bytes < L.w.total)
+    return fail(PKH3_EWORKSPACE, "workspace too small: %zu < %zu bytes", a->workspace_bytes, L.w.total);
+  if ((rc = run_kv_side(a, L, (hipStream_t)stream))) return rc;
   g_err[0] = 0;
   return PKH3_OK;
 }

@@ -71,10 +71,11 @@ def fill_args(
     q, k, v, out, *, q_norm_weight=None, k_norm_weight=None, norm_eps=1e-6, rope_q=None, rope_k=None,
     rope_mode=_lib.ROPE_NONE, key_mask=None, block_mask: Optional[BlockMask] = None, fp8_qk=False,
     softmax_scale: Optional[float] = None, long_key_kernel: bool = False, kv_prepared: bool = False,
-    out_images: bool = False,
+    out_images: bool = False, prepared_keys: Optional[int] = None,
 ) -> Tuple[_lib.AttnArgs, list]:
     """Build ``pkh3_attn_args`` for these tensors.  Returns (args, keep_alive).  ``kv_prepared``: K and V
-    come from the fused projection (``pkh3_qkv_proj``) through the workspace; ``k`` and ``v`` are then None.
+    come through the workspace, from the fused projection (``pkh3_qkv_proj``) or from ``pkh3_kv_prepare``
+    (then ``prepared_keys`` is their Sk); ``k`` and ``v`` are then None.
     ``out_images``: ``out`` is a uint8 operand-image buffer for ``pkh3_out_proj`` (``projections.packed_bytes(Sq,
     H*D)`` bytes) instead of a ``[B, Sq, H, D]`` tensor, and B must be 1."""
     if kv_prepared != (k is None) or (k is None) != (v is None):
@@ -83,7 +84,7 @@ def fill_args(
         if t is not None:
             _check_bshd(n, t)
     B, Sq, H, D = q.shape
-    Sk = Sq if k is None else k.shape[1]
+    Sk = (Sq if prepared_keys is None else int(prepared_keys)) if k is None else k.shape[1]
     if k is not None and (tuple(k.shape) != (B, Sk, H, D) or tuple(v.shape) != (B, Sk, H, D)):
         raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
     if out_images:
@@ -192,6 +193,72 @@ def attention(
         _lib.check(lib.pkh3_attn_fwd(C.byref(args), C.c_void_p(stream.cuda_stream)))
         # the workspace must outlive the kernels: tie it to the stream, not to this Python frame
         workspace.record_stream(stream)
+    return out
+
+
+@dataclass
+class PreparedKV:
+    """Keys and values of :func:`prepare_kv`, ready for any number of :func:`attention` calls."""
+
+    workspace: torch.Tensor  # holds K', V, scales, row-norm maxima and the compacted key list
+    B: int
+    Sk: int
+    H: int
+    opts: dict               # the K-side options every later call must repeat
+
+
+K_SIDE_OPTIONS = ("k_norm_weight", "norm_eps", "rope_k", "rope_mode", "key_mask", "fp8_qk")
+
+
+def prepare_kv(k: torch.Tensor, v: torch.Tensor, *, q_rows: Optional[int] = None, **opts) -> PreparedKV:
+    """The K/V side of :func:`attention` on its own (``pkh3_kv_prepare``): for keys and values several calls
+    share, e.g. the text keys of a block's cross-attention over the denoising steps.  ``opts``: ``k_norm_weight``,
+    ``norm_eps``, ``rope_mode`` + ``rope_k``, ``key_mask``, ``fp8_qk``.  ``q_rows``: the largest query count of the
+    calls that will follow (default Sk); dense calls need no more scratch than the K/V side itself."""
+    lib = _lib.load()
+    unknown = set(opts) - set(K_SIDE_OPTIONS)
+    if unknown:
+        raise ValueError(f"prepare_kv takes the K-side options {K_SIDE_OPTIONS}, got {sorted(unknown)}")
+    _check_bshd("k", k)
+    B, Sk, H, D = k.shape
+    full = dict(opts)
+    if full.get("rope_mode", _lib.ROPE_NONE) != _lib.ROPE_NONE:
+        full["rope_q"] = full.get("rope_k")  # the call validates four tables; the Q pair is not read here
+    # a stand-in for q and o with the right shape and device (one row of storage): this entry point reads neither
+    stand_in = torch.empty((1, 1, 1, D), dtype=k.dtype, device=k.device).expand(B, Sk, H, D)
+    args, keep = fill_args(stand_in, k, v, stand_in, **full)
+    args.Sq = int(q_rows or Sk)
+    ws = torch.empty(workspace_bytes(args), dtype=torch.uint8, device=k.device)
+    args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+    args.q = args.o = None
+    with torch.cuda.device(k.device):
+        _lib.check(lib.pkh3_kv_prepare(C.byref(args), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    return PreparedKV(ws, int(B), int(Sk), int(H), dict(opts))
+
+
+def attention_prepared(q: torch.Tensor, kv: PreparedKV, *, out: Optional[torch.Tensor] = None, **q_opts) -> torch.Tensor:
+    """:func:`attention` of ``q`` against prepared keys and values.  ``q_opts``: the Q-side options
+    (``q_norm_weight``, ``rope_q``, ``softmax_scale``, ``long_key_kernel``); the K-side ones come from ``kv``."""
+    lib = _lib.load()
+    clash = set(q_opts) & set(K_SIDE_OPTIONS)
+    if clash:
+        raise ValueError(f"K-side options belong to prepare_kv: {sorted(clash)}")
+    if out is None:
+        out = torch.empty_like(q)
+    opts = dict(kv.opts)
+    opts.update(q_opts)
+    args, keep = fill_args(q, None, None, out, kv_prepared=True, prepared_keys=kv.Sk, **opts)
+    if (args.B, args.H) != (kv.B, kv.H):
+        raise ValueError(f"q has batch {args.B} and {args.H} heads, the prepared keys {kv.B} and {kv.H}")
+    _on_device("prepared workspace", kv.workspace, q.device)
+    need = workspace_bytes(args)
+    if kv.workspace.numel() < need:
+        raise ValueError(f"the prepared workspace holds {kv.workspace.numel()} bytes, this call needs {need} (give prepare_kv q_rows)")
+    args.workspace, args.workspace_bytes = kv.workspace.data_ptr(), kv.workspace.numel()
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream()
+        _lib.check(lib.pkh3_attn_fwd(C.byref(args), C.c_void_p(stream.cuda_stream)))
+        kv.workspace.record_stream(stream)
     return out
 
 

@@ -22,7 +22,7 @@ def test_header_symbols_are_exported(lib):
 
 
 def test_version_and_strerror(lib):
-    assert lib.pkh3_version() == 104
+    assert lib.pkh3_version() == 105
     assert lib.pkh3_strerror(0) == b"ok"
     assert b"128" in lib.pkh3_strerror(_lib.PKH3_EHEADDIM)
 
@@ -259,13 +259,36 @@ def test_qkv_proj_argument_errors(lib):
     assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_EWORKSPACE
     p, a = _qkv_args(); a.workspace_bytes = 1024
     assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_EWORKSPACE
-    # the attention call on prepared K/V: k and v may be NULL, but the shape restrictions stay
+    # the attention call on prepared K/V: k and v may be NULL only with the flag; the fused projection itself keeps
+    # its one-document restriction, and the entry point without a workspace cannot take prepared K/V at all
     p, a = _qkv_args(); a.k = a.v = 0
     assert lib.pkh3_attn_fwd(C.byref(a), None) == _lib.PKH3_ENULL
-    a.flags = _lib.FLAG_KV_PREPARED; a.B = 2
-    assert lib.pkh3_attn_fwd(C.byref(a), None) == _lib.PKH3_EUNSUPPORTED
-    a.B = 1
+    a.flags = _lib.FLAG_KV_PREPARED
     assert lib.pkh3_attn_fwd_noalloc(C.byref(a), None) == _lib.PKH3_EUNSUPPORTED
+    a.B = 2
+    assert lib.pkh3_qkv_proj(C.byref(p), C.byref(a), None) == _lib.PKH3_EUNSUPPORTED
+
+
+def test_kv_prepare_argument_errors(lib):
+    """The K/V side alone: q and o are not looked at, everything else is checked as in the attention call."""
+    a = _valid_args()
+    a.q = a.o = 0
+    a.k = 0
+    assert lib.pkh3_kv_prepare(C.byref(a), None) == _lib.PKH3_ENULL
+    a = _valid_args(); a.q = a.o = 0; a.workspace_bytes = 1024
+    assert lib.pkh3_kv_prepare(C.byref(a), None) == _lib.PKH3_EWORKSPACE
+    a = _valid_args(); a.q = a.o = 0; a.flags = _lib.FLAG_KV_PREPARED
+    assert lib.pkh3_kv_prepare(C.byref(a), None) == _lib.PKH3_EARG
+    a = _valid_args(); a.q = a.o = 0; a.v_ss = 132
+    assert lib.pkh3_kv_prepare(C.byref(a), None) == _lib.PKH3_ESTRIDE
+    assert lib.pkh3_kv_prepare(None, None) == _lib.PKH3_ENULL
+    # the K/V side of the workspace does not move with the queries or the block map of the later calls
+    a = _valid_args()
+    dense = lib.pkh3_workspace_bytes(C.byref(a))
+    a.Sq = 100000
+    assert lib.pkh3_workspace_bytes(C.byref(a)) == dense
+    a.blk_row_ptr, a.blk_col_idx = 0x20000, 0x30000
+    assert lib.pkh3_workspace_bytes(C.byref(a)) > dense
 
 
 def test_out_proj_argument_errors(lib):

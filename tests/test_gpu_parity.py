@@ -233,3 +233,40 @@ def test_hip_graph_replays_match_eager(variant):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {rep} differs from the eager call"
+
+
+@pytest.mark.parametrize("variant", ["cross_masked", "rope_fp8", "long_keys"])
+def test_prepared_keys_serve_several_calls(variant):
+    """pkh3_kv_prepare once, then attention calls with different queries (and query counts) on the prepared
+    workspace: each must give the bits of the ordinary call on the same q, k, v."""
+    import pika_h3_flex_amd as pk
+
+    gen = torch.Generator().manual_seed(17)
+    dev = "cuda"
+    B, H, D = (2, 2, 128) if variant == "cross_masked" else (1, 3, 128)
+    Sk = {"cross_masked": 100, "rope_fp8": 333, "long_keys": 1500}[variant]
+    k, v = (_rand((B, Sk, H, D), gen).to(dev) for _ in range(2))
+    wq = (1.0 + 0.1 * torch.randn(D, generator=gen)).to(dev)
+    wk = (1.0 + 0.1 * torch.randn(D, generator=gen)).to(dev)
+    k_opts = dict(k_norm_weight=wk)
+    if variant == "cross_masked":
+        k_opts.update(key_mask=(torch.rand((B, Sk), generator=gen) < 0.6).to(dev))
+    tabs_k = None
+    if variant == "rope_fp8":
+        tabs_k = pk.rope_tables((torch.rand((Sk, 3), generator=gen, dtype=torch.float64) * 20).to(dev))
+        k_opts.update(rope_mode=pk.ROPE_INTERLEAVED, rope_k=tabs_k, fp8_qk=True)
+    kv = pk.prepare_kv(k, v, q_rows=700, **k_opts)
+    for Sq in (77, 700, 300):
+        q = _rand((B, Sq, H, D), gen).to(dev)
+        q_opts = dict(q_norm_weight=wq)
+        if variant == "rope_fp8":
+            q_opts.update(rope_q=pk.rope_tables((torch.rand((Sq, 3), generator=gen, dtype=torch.float64) * 20).to(dev)))
+        got = pk.attention_prepared(q, kv, **q_opts)
+        want = pk.attention(q, k, v, **k_opts, **q_opts)
+        torch.cuda.synchronize()
+        assert torch.isfinite(got.float()).all()
+        assert torch.equal(got, want), f"{variant} Sq={Sq}: prepared keys give different bits"
+    with pytest.raises(ValueError, match="K-side"):
+        pk.attention_prepared(q, kv, k_norm_weight=wk, **q_opts)
+    with pytest.raises(ValueError, match="heads"):
+        pk.attention_prepared(_rand((B, Sq, H + 1, D), gen).to(dev), kv, **q_opts)
