@@ -19,7 +19,7 @@ from typing import Dict, Hashable, Optional, Tuple
 import torch
 
 from . import _lib
-from .ops import BlockMask, attention, rope_tables
+from .ops import BlockMask, PreparedKV, attention, attention_prepared, prepare_kv, rope_tables
 from .projections import PackedLinear, adaln_modulate, out_proj, pack_rows, qkv_attention
 
 
@@ -52,6 +52,7 @@ class PikaH3AttnProcessor:
         fp8_qk: bool = False,
         fused_projections: bool = False,
         lora_adapter: str = "default",
+        cache_cross_kv: bool = False,
     ):
         self.rope_mode = int(rope_mode)
         self.rope_axes_dims = tuple(int(x) for x in rope_axes_dims)
@@ -62,6 +63,11 @@ class PikaH3AttnProcessor:
         # K/V written by the GEMM epilogue in the attention kernel's layout) instead of the module's torch GEMMs
         self.fused_projections = bool(fused_projections)
         self.lora_adapter = str(lora_adapter)
+        # cross-attention: the text keys and values of a block are the same in every denoising step of a clip (the
+        # model runs six times on one prompt, src/pika_h3/pipeline.py:13); with this switch a block projects and
+        # prepares them once per (module, encoder_hidden_states tensor, mask tensor) and later steps reuse them
+        self.cache_cross_kv = bool(cache_cross_kv)
+        self._cross_kv: Dict[Hashable, Tuple[tuple, PreparedKV]] = {}
         self._packed: Dict[int, Tuple[object, Dict[str, PackedLinear]]] = {}
         # position grids are constant across layers and denoising steps: one table per grid
         self._rope_cache: Dict[Hashable, Tuple[Optional[torch.Tensor], Tuple[torch.Tensor, torch.Tensor]]] = {}
@@ -112,11 +118,33 @@ class PikaH3AttnProcessor:
         return hit[1]
 
     def forget(self, attn=None) -> None:
-        """Drop packed weights (of one module, or all)."""
+        """Drop packed weights and prepared cross-attention keys (of one module, or all)."""
         if attn is None:
             self._packed.clear()
+            self._cross_kv.clear()
         else:
             self._packed.pop(id(attn), None)
+            for key in [k for k in self._cross_kv if k[0] == id(attn)]:
+                del self._cross_kv[key]
+
+    def _prepared_cross_kv(self, attn, enc: torch.Tensor, mask: Optional[torch.Tensor], k_opts: dict, H: int) -> PreparedKV:
+        """Prepared K/V of ``attn``'s cross-attention over ``enc``: keyed by the module and by the identity and
+        in-place version of the two tensors, which the entry keeps alive (so their addresses cannot be reused)."""
+        key = (id(attn), enc.data_ptr(), enc._version, tuple(enc.shape), str(enc.device),
+               None if mask is None else (mask.data_ptr(), mask._version), float(k_opts["norm_eps"]), bool(k_opts["fp8_qk"]))
+        hit = self._cross_kv.get(key)
+        if hit is not None and hit[0][0] is attn and hit[0][1] is enc and hit[0][2] is mask:
+            return hit[1]
+        B, Sk, _ = enc.shape
+        k = attn.to_k(enc).view(B, Sk, H, -1)
+        v = attn.to_v(enc).view(B, Sk, H, -1)
+        if k.dtype != torch.bfloat16:
+            k, v = k.to(torch.bfloat16), v.to(torch.bfloat16)
+        kv = prepare_kv(k, v, **k_opts)
+        if len(self._cross_kv) >= 256:
+            self._cross_kv.pop(next(iter(self._cross_kv)))
+        self._cross_kv[key] = ((attn, enc, mask), kv)
+        return kv
 
     def __call__(
         self,
@@ -161,23 +189,31 @@ class PikaH3AttnProcessor:
         if fused:
             return self._fused(attn, hidden_states, position_ids=position_ids, rope_cos_sin=rope_cos_sin, block_mask=block_mask,
                                fp8_qk=fp8_qk, rope_key=rope_key, adaln=adaln, gate=gate, gate_index=gate_index, residual=residual)
-        kv_src = hidden_states if encoder_hidden_states is None else encoder_hidden_states
-        q = attn.to_q(hidden_states)
-        k = attn.to_k(kv_src)
-        v = attn.to_v(kv_src)
-        D = q.shape[-1] // H
-        # [B, S, H*D] -> [B, S, H, D] views: no transpose copy, the kernels take the strides
-        q = q.view(B, S, H, D)
-        k = k.view(B, kv_src.shape[1], H, D)
-        v = v.view(B, kv_src.shape[1], H, D)
-        if q.dtype != torch.bfloat16:
-            q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
-
         qn, kn = getattr(attn, "norm_q", None), getattr(attn, "norm_k", None)
         eps = getattr(qn, "eps", None)
         eps = self.norm_eps if eps is None else float(eps)
         scale = getattr(attn, "scale", None)
         use_fp8 = (self.fp8_qk if fp8_qk is None else bool(fp8_qk)) and attention_mask is None
+        q = attn.to_q(hidden_states)
+        D = q.shape[-1] // H
+        # [B, S, H*D] -> [B, S, H, D] views: no transpose copy, the kernels take the strides
+        q = q.view(B, S, H, D)
+        if q.dtype != torch.bfloat16:
+            q = q.to(torch.bfloat16)
+        if encoder_hidden_states is not None and self.cache_cross_kv and block_mask is None:
+            k_opts = dict(k_norm_weight=_norm_weight(kn, D, q.device), norm_eps=eps, fp8_qk=use_fp8)
+            if attention_mask is not None:
+                k_opts.update(key_mask=attention_mask)
+            kv = self._prepared_cross_kv(attn, encoder_hidden_states, attention_mask, k_opts, H)
+            out = attention_prepared(q, kv, q_norm_weight=_norm_weight(qn, D, q.device),
+                                     softmax_scale=None if scale is None else float(scale))
+            out = attn.to_out[0](out.view(B, S, H * D).to(hidden_states.dtype))
+            return attn.to_out[1](out) if len(attn.to_out) > 1 else out
+        kv_src = hidden_states if encoder_hidden_states is None else encoder_hidden_states
+        k = attn.to_k(kv_src).view(B, kv_src.shape[1], H, D)
+        v = attn.to_v(kv_src).view(B, kv_src.shape[1], H, D)
+        if k.dtype != torch.bfloat16:
+            k, v = k.to(torch.bfloat16), v.to(torch.bfloat16)
         opts = dict(
             q_norm_weight=_norm_weight(qn, D, q.device),
             k_norm_weight=_norm_weight(kn, D, q.device),

@@ -370,6 +370,42 @@ def test_processor_self_and_cross():
 
 
 @pytest.mark.gpu
+def test_processor_prepares_cross_attention_keys_once():
+    """cache_cross_kv: a block's text keys and values are projected and prepared on the first call and read again by
+    the later denoising steps (new queries, same encoder states); an in-place change of the encoder states, another
+    tensor or `forget` prepare them anew.  Results equal the uncached processor's bit for bit."""
+    import pika_h3_flex_amd as pk
+
+    torch.manual_seed(5)
+    H, hidden, S, Sk = 3, 384, 150, 64
+    attn = _Attn(hidden, H, kv_dim=200).cuda().to(torch.bfloat16)
+    calls = {"k": 0}
+    attn.to_k.register_forward_hook(lambda *_: calls.__setitem__("k", calls["k"] + 1))
+    enc = torch.randn((1, Sk, 200), device="cuda", dtype=torch.bfloat16)
+    mask = (torch.arange(Sk, device="cuda") < 23)[None, :]
+    plain, cached = pk.PikaH3AttnProcessor(), pk.PikaH3AttnProcessor(cache_cross_kv=True)
+    with torch.no_grad():
+        for step in range(3):
+            x = torch.randn((1, S + 10 * step, hidden), device="cuda", dtype=torch.bfloat16)
+            want = plain(attn, x, encoder_hidden_states=enc, attention_mask=mask)
+            before = calls["k"]
+            got = cached(attn, x, encoder_hidden_states=enc, attention_mask=mask)
+            torch.cuda.synchronize()
+            assert calls["k"] - before == (1 if step == 0 else 0), f"step {step}: to_k ran {calls['k'] - before} times"
+            assert torch.equal(got, want), f"step {step}"
+        enc.mul_(0.5)  # in place: the version counter moves, the keys are prepared again
+        before = calls["k"]
+        got = cached(attn, x, encoder_hidden_states=enc, attention_mask=mask)
+        assert calls["k"] - before == 1
+        assert torch.equal(got, plain(attn, x, encoder_hidden_states=enc, attention_mask=mask))
+        cached.forget(attn)
+        before = calls["k"]
+        cached(attn, x, encoder_hidden_states=enc)  # no mask: its own entry
+        cached(attn, x, encoder_hidden_states=enc)
+        assert calls["k"] - before == 1
+
+
+@pytest.mark.gpu
 def test_processor_on_a_packed_document():
     """One packed document (text, keyframe rows, audio, video) built from latents by the packing helpers:
     the processor with the layout's positions against the oracle on the same rows."""
