@@ -210,11 +210,13 @@ class PreparedKV:
 K_SIDE_OPTIONS = ("k_norm_weight", "norm_eps", "rope_k", "rope_mode", "key_mask", "fp8_qk")
 
 
-def prepare_kv(k: torch.Tensor, v: torch.Tensor, *, q_rows: Optional[int] = None, **opts) -> PreparedKV:
+def prepare_kv(k: torch.Tensor, v: torch.Tensor, *, q_rows: Optional[int] = None, block_sparse: bool = False,
+               **opts) -> PreparedKV:
     """The K/V side of :func:`attention` on its own (``pkh3_kv_prepare``): for keys and values several calls
     share, e.g. the text keys of a block's cross-attention over the denoising steps.  ``opts``: ``k_norm_weight``,
-    ``norm_eps``, ``rope_mode`` + ``rope_k``, ``key_mask``, ``fp8_qk``.  ``q_rows``: the largest query count of the
-    calls that will follow (default Sk); dense calls need no more scratch than the K/V side itself."""
+    ``norm_eps``, ``rope_mode`` + ``rope_k``, ``key_mask``, ``fp8_qk``.  Dense calls need no more scratch than the
+    K/V side itself; when calls with a ``block_mask`` will follow, say so (``block_sparse=True``) and give the largest
+    query count among them (``q_rows``, default Sk), so that the workspace has room for their tile lists."""
     lib = _lib.load()
     unknown = set(opts) - set(K_SIDE_OPTIONS)
     if unknown:
@@ -228,7 +230,13 @@ def prepare_kv(k: torch.Tensor, v: torch.Tensor, *, q_rows: Optional[int] = None
     stand_in = torch.empty((1, 1, 1, D), dtype=k.dtype, device=k.device).expand(B, Sk, H, D)
     args, keep = fill_args(stand_in, k, v, stand_in, **full)
     args.Sq = int(q_rows or Sk)
-    ws = torch.empty(workspace_bytes(args), dtype=torch.uint8, device=k.device)
+    need = workspace_bytes(args)
+    if block_sparse:
+        # size with a block map present (only the pointers' presence matters to the sizing call)
+        args.blk_row_ptr = args.blk_col_idx = k.data_ptr()
+        need = workspace_bytes(args)
+        args.blk_row_ptr = args.blk_col_idx = None
+    ws = torch.empty(need, dtype=torch.uint8, device=k.device)
     args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
     args.q = args.o = None
     with torch.cuda.device(k.device):

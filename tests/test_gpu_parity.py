@@ -235,7 +235,7 @@ def test_hip_graph_replays_match_eager(variant):
         assert torch.equal(out, eager), f"replay {rep} differs from the eager call"
 
 
-@pytest.mark.parametrize("variant", ["cross_masked", "rope_fp8", "long_keys"])
+@pytest.mark.parametrize("variant", ["cross_masked", "rope_fp8", "long_keys", "block_sparse"])
 def test_prepared_keys_serve_several_calls(variant):
     """pkh3_kv_prepare once, then attention calls with different queries (and query counts) on the prepared
     workspace: each must give the bits of the ordinary call on the same q, k, v."""
@@ -244,7 +244,7 @@ def test_prepared_keys_serve_several_calls(variant):
     gen = torch.Generator().manual_seed(17)
     dev = "cuda"
     B, H, D = (2, 2, 128) if variant == "cross_masked" else (1, 3, 128)
-    Sk = {"cross_masked": 100, "rope_fp8": 333, "long_keys": 1500}[variant]
+    Sk = {"cross_masked": 100, "rope_fp8": 333, "long_keys": 1500, "block_sparse": 700}[variant]
     k, v = (_rand((B, Sk, H, D), gen).to(dev) for _ in range(2))
     wq = (1.0 + 0.1 * torch.randn(D, generator=gen)).to(dev)
     wk = (1.0 + 0.1 * torch.randn(D, generator=gen)).to(dev)
@@ -255,10 +255,13 @@ def test_prepared_keys_serve_several_calls(variant):
     if variant == "rope_fp8":
         tabs_k = pk.rope_tables((torch.rand((Sk, 3), generator=gen, dtype=torch.float64) * 20).to(dev))
         k_opts.update(rope_mode=pk.ROPE_INTERLEAVED, rope_k=tabs_k, fp8_qk=True)
-    kv = pk.prepare_kv(k, v, q_rows=700, **k_opts)
+    kv = pk.prepare_kv(k, v, q_rows=700, block_sparse=(variant == "block_sparse"), **k_opts)
     for Sq in (77, 700, 300):
         q = _rand((B, Sq, H, D), gen).to(dev)
         q_opts = dict(q_norm_weight=wq)
+        if variant == "block_sparse":  # every call brings its own tile map
+            tm = torch.rand(((Sq + 63) // 64, (Sk + 63) // 64), generator=gen) < 0.5
+            q_opts.update(block_mask=pk.BlockMask.from_dense(tm, device=dev))
         if variant == "rope_fp8":
             q_opts.update(rope_q=pk.rope_tables((torch.rand((Sq, 3), generator=gen, dtype=torch.float64) * 20).to(dev)))
         got = pk.attention_prepared(q, kv, **q_opts)
