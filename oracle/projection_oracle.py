@@ -16,6 +16,9 @@ Pinning status (tests/test_projection_oracle.py):
                   W + s B A (the identity PEFT's merge relies on), zero adapter, rank-one closed form
   adaln_modulate  pinned: torch.nn.functional.layer_norm / rms_norm, index_select, zero-modulation identity,
                   per-row constant closed form
+  modulation_tables  pinned: torch.nn.functional.silu in float32 + torch.nn.functional.linear; one rounding of
+                  the activation against a two-rounding evaluation, row order of the view checked against an
+                  explicit (timestep, modality) loop
   attention_block composition of the above with attention_oracle.reference_layer; pinned by its parts and
                   by an explicit per-row, per-head loop on a tiny case
 """
@@ -40,6 +43,19 @@ def lora_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
         down = x64 @ lora_a.to(device=x.device, dtype=torch.float64).t()
         y = y + float(lora_scale) * (down @ lora_b.to(device=x.device, dtype=torch.float64).t())
     return y
+
+
+def modulation_tables(temb: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], hidden_size: int,
+                      chunks: int = 6):
+    """patches/0001-h3-adaln-fp32.patch:126-133 restated: SiLU in float32 (``x * sigmoid(x)``, written out), the
+    result rounded to the projection's dtype, the linear layer in float64 on those rounded values, rows viewed as
+    ``[-1, chunks * hidden_size]`` and split.  Returns ``chunks`` float64 tables."""
+    t32 = temb.to(torch.float32)
+    act = (t32 * (1.0 / (1.0 + torch.exp(-t32)))).to(weight.dtype)
+    out = act.to(torch.float64) @ weight.to(torch.float64).t()
+    if bias is not None:
+        out = out + bias.to(torch.float64)
+    return tuple(out.view(-1, chunks * hidden_size).chunk(chunks, dim=-1))
 
 
 def adaln_modulate(x: torch.Tensor, *, shift: Optional[torch.Tensor] = None, scale: Optional[torch.Tensor] = None,

@@ -94,6 +94,41 @@ def adaln_modulate(x: torch.Tensor, *, shift: Optional[torch.Tensor] = None, sca
     return out
 
 
+def modulation_tables(temb: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], hidden_size: int,
+                      chunks: int = 6):
+    """The per-timestep modulation tables of a block, as the reference's patched module forms them
+    (patches/0001-h3-adaln-fp32.patch:126-133): ``linear(silu(temb.float()).to(weight.dtype))`` -- the activation
+    in float32 whatever dtype ``temb`` arrives in, only its result cast to the projection's dtype --, viewed as
+    ``[-1, chunks * hidden_size]`` and split into ``chunks`` tables ``[rows, hidden_size]`` (six for a block:
+    shift, scale, gate of the attention half and of the MLP half; two for the output norm, patch lines 150-158).
+    With several modalities behind one linear layer the rows come out timestep-major: row = timestep * modalities
+    + modality (see :func:`modulation_row_index`).  A few rows by a few thousand columns: host-side torch, the tables
+    are then inputs of :func:`adaln_modulate` (shift, scale) and :func:`out_proj` (gate)."""
+    if temb.dim() != 2 or weight.dim() != 2 or weight.shape[1] != temb.shape[1]:
+        raise ValueError(f"temb [rows, E] and weight [N, E] expected, got {tuple(temb.shape)} and {tuple(weight.shape)}")
+    if weight.shape[0] % (chunks * hidden_size):
+        raise ValueError(f"the layer has {weight.shape[0]} outputs, not a multiple of {chunks} x {hidden_size}")
+    act = torch.nn.functional.silu(temb.float()).to(weight.dtype)
+    out = torch.nn.functional.linear(act, weight, bias).view(-1, chunks * hidden_size)
+    return tuple(t.contiguous() for t in out.chunk(chunks, dim=-1))
+
+
+def modulation_row_index(timestep_indices: torch.Tensor, modality: Optional[torch.Tensor] = None, modalities: int = 1) -> torch.Tensor:
+    """int32 table row per token for :func:`adaln_modulate` / :func:`out_proj`: ``timestep_indices`` (the per-row
+    index of src/pika_h3/core/wrapper.py:182-190) alone, or ``timestep_indices * modalities + modality`` when the
+    tables of :func:`modulation_tables` hold one row per (timestep, modality).  Which chunk of the un-vendored
+    module belongs to which modality is not visible in the reference: ``modality`` is the caller's map from
+    ``token_tags`` (0 video, 1 text, 2 audio, src/pika_h3/core/geometry.py:40-42) to chunk numbers."""
+    idx = timestep_indices.to(torch.int64)
+    if modality is not None:
+        if modality.shape != timestep_indices.shape:
+            raise ValueError("modality must have one entry per row")
+        if int(modality.min()) < 0 or int(modality.max()) >= modalities:
+            raise ValueError(f"modality numbers must lie in [0, {modalities})")
+        idx = idx * int(modalities) + modality.to(idx.device, torch.int64)
+    return idx.to(torch.int32).contiguous()
+
+
 @dataclass
 class PackedLinear:
     """One linear layer, packed: ``y = x W^T + bias + lora_scale * (x A^T) B^T``."""

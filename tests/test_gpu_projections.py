@@ -350,7 +350,17 @@ def test_document_kwargs_drive_the_fused_block():
     attn = _Attn(hidden, H, True).cuda().to(torch.bfloat16)
     x = torch.randn((1, S, hidden), device="cuda", dtype=torch.bfloat16)      # the packed hidden states of the block
     K = times.numel()
-    shift, scale, gate = (torch.randn((K, hidden), device="cuda").mul(0.2).to(torch.bfloat16) for _ in range(3))
+    # the block's modulation tables from a time embedding per row time, the way the patched module forms them
+    # (float32 SiLU, then the linear layer; patches/0001-h3-adaln-fp32.patch:126-133): six tables of K rows
+    from pika_h3_flex_amd import projections as PR
+    temb = torch.randn((K, 64), device="cuda").to(torch.bfloat16)
+    mod_w = torch.randn((6 * hidden, 64), device="cuda").mul(0.03).to(torch.bfloat16)
+    mod_b = torch.randn(6 * hidden, device="cuda").mul(0.05).to(torch.bfloat16)
+    shift, scale, gate, _, _, _ = PR.modulation_tables(temb, mod_w, mod_b, hidden)
+    want = PO.modulation_tables(temb.cpu(), mod_w.cpu(), mod_b.cpu(), hidden)
+    for got_t, want_t in zip((shift, scale, gate), want):
+        assert float((got_t.cpu().double() - want_t).abs().max()) <= 2.0 ** -7 * max(1.0, float(want_t.abs().max()))
+    assert torch.equal(PR.modulation_row_index(tidx), tidx)
     proc = pk.PikaH3AttnProcessor(fused_projections=True)
     with torch.no_grad():
         y = proc(attn, x, position_ids=pos, adaln=dict(shift=shift, scale=scale, row_index=tidx, norm="layer"),

@@ -106,3 +106,54 @@ def test_attention_block_is_the_composition_of_its_parts():
                                  q_norm_weight=w, k_norm_weight=w)
     err, cos = AO.max_abs_and_cosine(rounded["y"], y)
     assert err < 2e-2 and cos > 0.9999
+
+
+def test_modulation_tables_activate_in_float32():
+    """patches/0001-h3-adaln-fp32.patch:126-133: SiLU in float32 whatever dtype temb arrives in, then the cast, then
+    the linear layer; rows of the view are (timestep, modality) pairs, timestep-major."""
+    from pika_h3_flex_amd import projections as P
+
+    g = torch.Generator().manual_seed(3)
+    T, E, hidden, M = 3, 64, 32, 2
+    temb = (torch.randn((T, E), generator=g) * 3).to(torch.bfloat16)
+    weight = (torch.randn((6 * hidden * M, E), generator=g) * 0.1).to(torch.bfloat16)
+    bias = (torch.randn(6 * hidden * M, generator=g) * 0.1).to(torch.bfloat16)
+    ref = PO.modulation_tables(temb, weight, bias, hidden)
+    # the library routine for the activation, in float32, agrees with the written-out form
+    lib = torch.nn.functional.linear(torch.nn.functional.silu(temb.float()).to(torch.bfloat16).double(), weight.double(), bias.double())
+    assert torch.allclose(torch.cat(ref, -1).reshape(T, -1), lib, atol=1e-12)
+    # the activation is monotone in precision: taken on float32 input it is at least as close to the float64 value
+    # as any bfloat16 evaluation can be (this torch build's bfloat16 SiLU already computes in float32 and rounds
+    # once, so on it the patch changes no bit; an evaluation that rounds the sigmoid first does differ)
+    exact = temb.double() * torch.sigmoid(temb.double())
+    one_rounding = torch.nn.functional.silu(temb.float()).to(torch.bfloat16).double()
+    two_roundings = (temb * torch.sigmoid(temb.float()).to(torch.bfloat16)).double()
+    assert float((one_rounding - exact).abs().max()) <= float((two_roundings - exact).abs().max())
+    assert float((one_rounding - two_roundings).abs().max()) > 0.0
+    got = P.modulation_tables(temb, weight, bias, hidden)
+    assert len(got) == 6 and all(t.shape == (T * M, hidden) and t.dtype == torch.bfloat16 for t in got)
+    for a, b in zip(got, ref):
+        assert float((a.double() - b).abs().max()) <= 2.0 ** -7 * max(1.0, float(b.abs().max()))  # one bf16 rounding of the output
+    # row order: row t*M + m of chunk c is the slice [(m*6 + c)*hidden, +hidden) of timestep t's output
+    for t in range(T):
+        for m in range(M):
+            for c in range(6):
+                want = lib[t, (m * 6 + c) * hidden:(m * 6 + c + 1) * hidden]
+                assert torch.equal(ref[c][t * M + m], want)
+    # two chunks: the output norm's table (patch lines 150-158)
+    assert len(P.modulation_tables(temb, weight[: 2 * hidden], bias[: 2 * hidden], hidden, chunks=2)) == 2
+    with pytest.raises(ValueError):
+        P.modulation_tables(temb, weight[:100], None, hidden)
+
+
+def test_modulation_row_index():
+    from pika_h3_flex_amd import projections as P
+
+    ti = torch.tensor([0, 0, 2, 1, 2])
+    assert P.modulation_row_index(ti).tolist() == [0, 0, 2, 1, 2] and P.modulation_row_index(ti).dtype == torch.int32
+    mod = torch.tensor([1, 0, 0, 2, 1])
+    assert P.modulation_row_index(ti, mod, 3).tolist() == [1, 0, 6, 5, 7]
+    with pytest.raises(ValueError):
+        P.modulation_row_index(ti, torch.tensor([0, 0, 3, 0, 0]), 3)
+    with pytest.raises(ValueError):
+        P.modulation_row_index(ti, mod[:3], 3)
