@@ -35,6 +35,30 @@ def _norm_weight(mod, dim: int, device) -> Optional[torch.Tensor]:
     return w.detach().to(device=device, dtype=torch.float32).contiguous()
 
 
+def key_padding_mask(attention_mask: Optional[torch.Tensor], batch: int, keys: int) -> Optional[torch.Tensor]:
+    """The forms diffusers modules hand a key-padding mask around in, as the bool ``[B, Sk]`` (True = attend) the
+    library takes: bool or integer ``[B, Sk]``; additive float masks (0 = attend, a large negative number = drop) of
+    shape ``[B, Sk]``, ``[B, 1, Sk]`` or ``[B, 1, 1, Sk]``.  A mask that differs between the queries or the heads of
+    a batch entry is not a key-padding mask and is refused."""
+    if attention_mask is None:
+        return None
+    m = attention_mask
+    if m.dim() > 2:
+        if any(d != 1 for d in m.shape[1:-1]):
+            raise ValueError(f"attention_mask {tuple(m.shape)} varies over queries or heads; only key-padding masks "
+                             f"[B, Sk] (or broadcast forms of them) are supported")
+        m = m.reshape(m.shape[0], m.shape[-1])
+    if m.dim() != 2 or m.shape[-1] != keys or m.shape[0] not in (1, batch):
+        raise ValueError(f"attention_mask must be [B, Sk] = [{batch}, {keys}] or a broadcast form, got {tuple(attention_mask.shape)}")
+    if m.shape[0] != batch:
+        m = m.expand(batch, keys)
+    if m.is_floating_point():
+        m = m > -1.0  # additive form: 0 keeps a key, -inf / a large negative number drops it
+    elif m.dtype != torch.bool:
+        m = m != 0
+    return m
+
+
 class PikaH3AttnProcessor:
     """Drop-in attention processor backed by the gfx950 HIP kernels.
 
@@ -166,8 +190,8 @@ class PikaH3AttnProcessor:
         """``hidden_states [B, S, H*D]`` -> ``[B, S, H*D]``.
 
         Self-attention when ``encoder_hidden_states`` is None, else cross-attention with K/V from
-        ``encoder_hidden_states [B, Sk, C]`` and ``attention_mask`` a bool key-padding mask
-        ``[B, Sk]`` (True = attend).  RoPE applies to self-attention only, from ``position_ids
+        ``encoder_hidden_states [B, Sk, C]`` and ``attention_mask`` a key-padding mask: bool
+        ``[B, Sk]`` (True = attend) or one of the forms :func:`key_padding_mask` converts.  RoPE applies to self-attention only, from ``position_ids
         [S, 3]`` (or precomputed ``rope_cos_sin`` fp32 ``[S, D/2]`` tables); ``rope_key`` names the grid for the
         table cache (see :meth:`_tables`).  The softmax scale is ``attn.scale`` when the module has one, else
         ``1/sqrt(D)``.  fp8 QK^T is not defined together with a key mask: such a call runs in bf16.
@@ -183,6 +207,11 @@ class PikaH3AttnProcessor:
             raise ValueError(f"hidden_states must be [B, S, C], got {tuple(hidden_states.shape)}")
         B, S, _ = hidden_states.shape
         H = int(attn.heads)
+        mask_given = attention_mask  # the caller's tensor: what the cross-attention key cache recognises
+        if attention_mask is not None:
+            keys = S if encoder_hidden_states is None else encoder_hidden_states.shape[1]
+            same = attention_mask.dtype == torch.bool and tuple(attention_mask.shape) == (B, keys)
+            attention_mask = attention_mask if same else key_padding_mask(attention_mask, B, keys)
         fused = self.fused_projections and encoder_hidden_states is None and attention_mask is None and B == 1
         if not fused and (adaln is not None or gate is not None or residual is not None):
             raise ValueError("adaln / gate / residual need fused_projections, self-attention, B = 1 and no mask")
@@ -204,7 +233,7 @@ class PikaH3AttnProcessor:
             k_opts = dict(k_norm_weight=_norm_weight(kn, D, q.device), norm_eps=eps, fp8_qk=use_fp8)
             if attention_mask is not None:
                 k_opts.update(key_mask=attention_mask)
-            kv = self._prepared_cross_kv(attn, encoder_hidden_states, attention_mask, k_opts, H)
+            kv = self._prepared_cross_kv(attn, encoder_hidden_states, mask_given, k_opts, H)
             out = attention_prepared(q, kv, q_norm_weight=_norm_weight(qn, D, q.device),
                                      softmax_scale=None if scale is None else float(scale))
             out = attn.to_out[0](out.view(B, S, H * D).to(hidden_states.dtype))

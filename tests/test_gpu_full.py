@@ -393,6 +393,13 @@ def test_processor_prepares_cross_attention_keys_once():
             torch.cuda.synchronize()
             assert calls["k"] - before == (1 if step == 0 else 0), f"step {step}: to_k ran {calls['k'] - before} times"
             assert torch.equal(got, want), f"step {step}"
+        # the additive form of the same mask (0 keeps a key, -inf drops it), as diffusers modules pass it around
+        additive = torch.zeros((1, 1, 1, Sk), device="cuda", dtype=torch.bfloat16).masked_fill(~mask[:, None, None, :], float("-inf"))
+        assert torch.equal(plain(attn, x, encoder_hidden_states=enc, attention_mask=additive), want)
+        before = calls["k"]
+        assert torch.equal(cached(attn, x, encoder_hidden_states=enc, attention_mask=additive), want)
+        assert torch.equal(cached(attn, x, encoder_hidden_states=enc, attention_mask=additive), want)
+        assert calls["k"] - before == 1  # its own cache entry, prepared once
         enc.mul_(0.5)  # in place: the version counter moves, the keys are prepared again
         before = calls["k"]
         got = cached(attn, x, encoder_hidden_states=enc, attention_mask=mask)

@@ -105,3 +105,21 @@ def test_processor_rejects_bad_input_and_host_tensors():
     # on a CPU tensor the processor must fail (no CPU fallback), after running the module's own projections
     with pytest.raises(ValueError, match="device memory"):
         proc(attn, torch.zeros((1, 4, 256), dtype=torch.bfloat16))
+
+
+def test_key_padding_mask_forms():
+    from pika_h3_flex_amd.processor import key_padding_mask
+
+    keep = torch.tensor([[True, True, False, False, True], [True, False, False, False, False]])
+    additive = torch.zeros((2, 5)).masked_fill(~keep, float("-inf"))
+    assert key_padding_mask(None, 2, 5) is None
+    assert torch.equal(key_padding_mask(keep, 2, 5), keep)
+    assert torch.equal(key_padding_mask(keep.to(torch.int64), 2, 5), keep)
+    assert torch.equal(key_padding_mask(additive, 2, 5), keep)
+    assert torch.equal(key_padding_mask(additive.to(torch.bfloat16)[:, None, None, :], 2, 5), keep)
+    assert torch.equal(key_padding_mask((additive * 0 - 10000.0 * (~keep))[:, None, :], 2, 5), keep)
+    assert torch.equal(key_padding_mask(keep[:1], 2, 5), keep[:1].expand(2, 5))
+    with pytest.raises(ValueError, match="queries or heads"):
+        key_padding_mask(torch.zeros((2, 4, 7, 5)), 2, 5)
+    with pytest.raises(ValueError, match="broadcast form"):
+        key_padding_mask(keep, 2, 6)
