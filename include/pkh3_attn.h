@@ -40,7 +40,7 @@
 extern "C" {
 #endif
 
-#define PKH3_VERSION 105
+#define PKH3_VERSION 106
 
 enum {
   PKH3_OK = 0,
@@ -109,8 +109,14 @@ typedef struct pkh3_attn_args {
      every key is masked gets an all-zero output row. */
   const uint8_t* key_mask;
   /* block-sparse map over 64x64 (query x key) tiles in CSR form, shared by all batches and heads:
-     blk_row_ptr int32 [ceil(Sq/64)+1], blk_col_idx int32 [blk_row_ptr[last]], columns strictly
-     ascending within a row.  NULL = dense.  Rows with no tile get an all-zero output. */
+     blk_row_ptr int32 [ceil(Sq/64)+1], blk_col_idx int32 [blk_row_ptr[last]].  NULL = dense.  Rows
+     with no tile get an all-zero output.
+     Preconditions, NOT checked (the arrays live in device memory and are read by a kernel only):
+     blk_row_ptr[0] = 0, blk_row_ptr non-decreasing, every value at most the number of int32 entries
+     allocated behind blk_col_idx; columns in [0, ceil(Sk/64)), each at most once per row (any order;
+     the library sorts).  What a violation does: a column outside the range is ignored, a repeated
+     column counts once, a row whose end lies before its start is treated as empty; blk_row_ptr values
+     beyond the blk_col_idx allocation make the planning kernel read out of bounds. */
   const int32_t* blk_row_ptr;
   const int32_t* blk_col_idx;
   uint32_t flags;
@@ -148,6 +154,14 @@ int pkh3_kv_prepare(const pkh3_attn_args* a, void* stream);
    results as pkh3_attn_fwd. */
 #define PKH3_NOALLOC_SCRATCH_BYTES (64u << 20)
 int pkh3_attn_fwd_noalloc(const pkh3_attn_args* a, void* stream);
+
+/* Set-up of pkh3_attn_fwd_noalloc for the CURRENT device: looks up the address of that device's copy of the
+   built-in array and the device's CU count and keeps both.  The first pkh3_attn_fwd_noalloc call on a device does
+   the same by itself, but these look-ups are not stream operations and a stream capture in progress may refuse
+   them: a caller that captures pkh3_attn_fwd_noalloc into a HIP graph calls this once per device beforehand (or
+   makes one ordinary call first).  Allocates nothing, launches nothing.  Like the call it serves it has no
+   counterpart in the reference. */
+int pkh3_noalloc_init(void);
 
 /* Rotary tables from the packed layout's position grid (src/pika_h3/core/packing.py:128 position_ids
    [S,3] float64, device memory).  axis_dims[3] are the head-dim slices per (t,h,w) axis (sum = D,

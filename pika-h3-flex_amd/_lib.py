@@ -36,6 +36,7 @@ EXPORTS = (
     "pkh3_attn_fwd",
     "pkh3_kv_prepare",
     "pkh3_attn_fwd_noalloc",
+    "pkh3_noalloc_init",
     "pkh3_rope_tables",
     "pkh3_version",
     "pkh3_strerror",
@@ -135,6 +136,8 @@ def load() -> C.CDLL:
     lib.pkh3_kv_prepare.restype = C.c_int
     lib.pkh3_attn_fwd_noalloc.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
     lib.pkh3_attn_fwd_noalloc.restype = C.c_int
+    lib.pkh3_noalloc_init.argtypes = []
+    lib.pkh3_noalloc_init.restype = C.c_int
     lib.pkh3_attn_time_kernel.argtypes = [C.POINTER(AttnArgs), C.c_void_p, C.c_int, C.POINTER(C.c_float)]
     lib.pkh3_attn_time_kernel.restype = C.c_int
     lib.pkh3_rope_tables.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_int32), C.c_double, C.c_void_p, C.c_void_p, C.c_void_p]

@@ -322,6 +322,17 @@ int pkh3_kv_prepare(const pkh3_attn_args* a, void* stream) {
   return PKH3_OK;
 }
 
+int pkh3_noalloc_init(void) {
+  void* ptr = nullptr;
+  int rc = static_scratch(&ptr);
+  if (rc) return rc;
+  int cus = 0;
+  hipError_t e = device_cu_count(&cus);
+  if (e != hipSuccess) return hip_fail(e, "device properties");
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
 int pkh3_attn_fwd_noalloc(const pkh3_attn_args* a, void* stream) {
   int rc = validate(a, true, /*caller_workspace=*/false);
   if (rc) return rc;

@@ -817,8 +817,8 @@ static void launch_fp(const FwdParams& p, int cus, hipStream_t st) {
   }
 }
 
-hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
-  // CUs of the current device, asked once per device; threads that race here store the same value
+// CUs of the current device, asked once per device; threads that race here store the same value
+hipError_t device_cu_count(int* out) {
   static std::atomic<int> cu_count[64];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -832,6 +832,14 @@ hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
       cu_count[dev].store(cus, std::memory_order_relaxed);
     }
   }
+  *out = cus;
+  return hipSuccess;
+}
+
+hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
+  int cus = 0;
+  hipError_t e = device_cu_count(&cus);
+  if (e != hipSuccess) return e;
   if (p.fp8) launch_fp<true>(p, cus, st);
   else launch_fp<false>(p, cus, st);
   return hipGetLastError();
@@ -863,7 +871,8 @@ __global__ __launch_bounds__(256) void sparse_plan_kernel(const int* __restrict_
       const int beg = row_ptr[row], end = row_ptr[row + 1];
       for (int j = beg + tid; j < end; j += 256) {
         const int col = col_idx[j] - base;
-        // a row lists a column at most once, so within one r no two threads touch the same byte
+        // within one r two threads touch the same byte only when the row repeats a column, and then both store the
+        // same value; columns outside [0, nKt) are ignored; a row whose end lies before its start is empty
         if (col >= 0 && col < kPlanChunk && col + base < nKt) mask[col] |= (unsigned char)(1 << r);
       }
       __syncthreads();

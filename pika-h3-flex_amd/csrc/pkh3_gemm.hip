@@ -459,7 +459,7 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackParams p) {
   const bool valid = src < p.rows;
   const int pieces = p.K / 8;                        // 16-byte pieces per row
   float v[kPackMaxPieces][8];
-  float sum = 0.f, ssq = 0.f;
+  float sum = 0.f;
 #pragma unroll
   for (int c = 0; c < kPackMaxPieces; ++c) {
     const int pc = lane + 64 * c;
@@ -469,19 +469,27 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackParams p) {
     for (int j = 0; j < 8; ++j) {
       v[c][j] = (float)t[j];
       sum += v[c][j];
-      ssq += v[c][j] * v[c][j];
     }
   }
   if constexpr (NORM != kNormNone) {
+    // Two passes over the row held in registers: the mean first, then the sum of squared distances from it.  The
+    // one-pass form E[x^2] - mean^2 cancels when a row's mean is large against its spread.
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) {
-      sum += __shfl_xor(sum, o, 64);
-      ssq += __shfl_xor(ssq, o, 64);
-    }
+    for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
     const float inv_k = 1.0f / (float)p.K;
     const float mean = NORM == kNormLayer ? sum * inv_k : 0.f;
-    const float var = NORM == kNormLayer ? fmaxf(ssq * inv_k - mean * mean, 0.f) : ssq * inv_k;
-    const float rs = rsqrtf(var + p.eps);
+    float ssq = 0.f;
+#pragma unroll
+    for (int c = 0; c < kPackMaxPieces; ++c) {
+      if (lane + 64 * c >= pieces) continue;  // pieces past the row's end hold zeros, not elements
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ssq += (v[c][j] - mean) * (v[c][j] - mean);
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) ssq += __shfl_xor(ssq, o, 64);
+    // a constant row with eps == 0 comes out as zeros (plus shift) instead of 0 * inf
+    const float ve = ssq * inv_k + p.eps;
+    const float rs = ve > 0.f ? rsqrtf(ve) : 0.f;
     const int mrow = valid && p.row_index ? p.row_index[src] : 0;
     const __bf16* sh = p.shift ? (const __bf16*)p.shift + (int64_t)mrow * p.table_stride : nullptr;
     const __bf16* sc = p.scale ? (const __bf16*)p.scale + (int64_t)mrow * p.table_stride : nullptr;

@@ -163,6 +163,7 @@ hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int
 hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st);
 hipError_t launch_v_prologue(const VPrologueParams& p, hipStream_t st);
 hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st);
+hipError_t device_cu_count(int* out);  // CUs of the current device (cached per device after the first call)
 hipError_t launch_sparse_plan(const int* row_ptr, const int* col_idx, int nRow64, int nQ64, int nKt, int* plan,
                               int plan_stride, int* plan_cnt, hipStream_t st);
 hipError_t launch_rope_tables(const double* pos, int S, const int* axis_dims, double theta, float* cos_out,

@@ -196,6 +196,14 @@ def attention(
     return out
 
 
+def noalloc_init(device=None) -> None:
+    """Set-up of the ``static_scratch=True`` calls on ``device`` (default: the current one): ``pkh3_noalloc_init``.
+    Needed once per device before such a call is captured into a HIP graph; otherwise the first call does it."""
+    lib = _lib.load()
+    with torch.cuda.device(device if device is not None else torch.cuda.current_device()):
+        _lib.check(lib.pkh3_noalloc_init())
+
+
 @dataclass
 class PreparedKV:
     """Keys and values of :func:`prepare_kv`, ready for any number of :func:`attention` calls."""

@@ -23,6 +23,9 @@ from .ops import BlockMask, PreparedKV, attention, attention_prepared, prepare_k
 from .projections import PackedLinear, adaln_modulate, out_proj, pack_rows, qkv_attention
 
 
+ADDITIVE_DROP_THRESHOLD = -1e3  # additive float masks: entries at or below this drop the key
+
+
 def _norm_weight(mod, dim: int, device) -> Optional[torch.Tensor]:
     """fp32 weight of an RMSNorm-like module (``None`` module = no norm; no ``weight`` = ones)."""
     if mod is None:
@@ -37,7 +40,7 @@ def _norm_weight(mod, dim: int, device) -> Optional[torch.Tensor]:
 
 def key_padding_mask(attention_mask: Optional[torch.Tensor], batch: int, keys: int) -> Optional[torch.Tensor]:
     """The forms diffusers modules hand a key-padding mask around in, as the bool ``[B, Sk]`` (True = attend) the
-    library takes: bool or integer ``[B, Sk]``; additive float masks (0 = attend, a large negative number = drop) of
+    library takes: bool or integer ``[B, Sk]``; additive float masks (0 = attend, -inf or a number <= -1000 = drop; other values are refused) of
     shape ``[B, Sk]``, ``[B, 1, Sk]`` or ``[B, 1, 1, Sk]``.  A mask that differs between the queries or the heads of
     a batch entry is not a key-padding mask and is refused."""
     if attention_mask is None:
@@ -53,7 +56,15 @@ def key_padding_mask(attention_mask: Optional[torch.Tensor], batch: int, keys: i
     if m.shape[0] != batch:
         m = m.expand(batch, keys)
     if m.is_floating_point():
-        m = m > -1.0  # additive form: 0 keeps a key, -inf / a large negative number drops it
+        # additive form: 0 keeps a key, -inf / a large negative number drops it.  Anything else -- a {0, 1} keep-mask
+        # cast to float, a soft bias -- is not a key-padding mask; turning it into keep/drop silently would attend
+        # padding keys or drop a bias, so it is refused (one reduction and one host read per distinct mask tensor)
+        keep = m == 0
+        if not bool((keep | (m <= ADDITIVE_DROP_THRESHOLD)).all()):
+            raise ValueError("floating-point attention_mask must be additive with entries 0 (attend) or <= "
+                             f"{ADDITIVE_DROP_THRESHOLD:g} (drop); got other values (a 0/1 keep-mask must be bool or integer, "
+                             "a soft additive bias is not supported)")
+        m = keep
     elif m.dtype != torch.bool:
         m = m != 0
     return m
@@ -77,6 +88,7 @@ class PikaH3AttnProcessor:
         fused_projections: bool = False,
         lora_adapter: str = "default",
         cache_cross_kv: bool = False,
+        cross_kv_cache_bytes: int = 1 << 30,
     ):
         self.rope_mode = int(rope_mode)
         self.rope_axes_dims = tuple(int(x) for x in rope_axes_dims)
@@ -91,6 +103,7 @@ class PikaH3AttnProcessor:
         # model runs six times on one prompt, src/pika_h3/pipeline.py:13); with this switch a block projects and
         # prepares them once per (module, encoder_hidden_states tensor, mask tensor) and later steps reuse them
         self.cache_cross_kv = bool(cache_cross_kv)
+        self.cross_kv_cache_bytes = int(cross_kv_cache_bytes)  # prepared workspaces kept at most (oldest dropped first)
         self._cross_kv: Dict[Hashable, Tuple[tuple, PreparedKV]] = {}
         self._packed: Dict[int, Tuple[object, Dict[str, PackedLinear]]] = {}
         # position grids are constant across layers and denoising steps: one table per grid
@@ -151,13 +164,33 @@ class PikaH3AttnProcessor:
             for key in [k for k in self._cross_kv if k[0] == id(attn)]:
                 del self._cross_kv[key]
 
-    def _prepared_cross_kv(self, attn, enc: torch.Tensor, mask: Optional[torch.Tensor], k_opts: dict, H: int) -> PreparedKV:
-        """Prepared K/V of ``attn``'s cross-attention over ``enc``: keyed by the module and by the identity and
-        in-place version of the two tensors, which the entry keeps alive (so their addresses cannot be reused)."""
-        key = (id(attn), enc.data_ptr(), enc._version, tuple(enc.shape), str(enc.device),
-               None if mask is None else (mask.data_ptr(), mask._version), float(k_opts["norm_eps"]), bool(k_opts["fp8_qk"]))
+    @staticmethod
+    def _weights_state(attn) -> tuple:
+        """Identity and in-place version of every parameter the prepared keys depend on: ``to_k`` / ``to_v`` (adapter
+        weights of a LoRA wrapper included: they are sub-module parameters) and the K-side norm."""
+        state = []
+        for mod in (attn.to_k, attn.to_v, getattr(attn, "norm_k", None)):
+            if mod is not None and hasattr(mod, "parameters"):
+                state += [(id(p_), p_._version) for p_ in mod.parameters()]
+        return tuple(state)
+
+    def _prepared_cross_kv(self, attn, enc: torch.Tensor, mask: Optional[torch.Tensor], k_opts: dict, H: int,
+                           cache_key: Optional[Hashable] = None) -> PreparedKV:
+        """Prepared K/V of ``attn``'s cross-attention over ``enc``.  With ``cache_key`` (the caller's name for the
+        prompt, e.g. a request id) the entry is found by (module, key) whatever tensors carry the text states in this
+        step -- a model that re-projects or re-concatenates them per forward still hits.  Without it the entry is
+        keyed by the identity and in-place version of the two tensors, which it keeps alive (so their addresses
+        cannot be reused).  Either way the key also holds the identity and version of the module's K-side weights
+        (adapters included), so training steps or a swapped adapter prepare the keys again.  The cache is bounded by
+        the bytes of its workspaces (``cross_kv_cache_bytes``), oldest entries dropped first."""
+        common = (float(k_opts["norm_eps"]), bool(k_opts["fp8_qk"]), tuple(enc.shape), str(enc.device), self._weights_state(attn))
+        if cache_key is not None:
+            key = (id(attn), "key", cache_key) + common
+        else:
+            key = (id(attn), "tensor", enc.data_ptr(), enc._version,
+                   None if mask is None else (mask.data_ptr(), mask._version)) + common
         hit = self._cross_kv.get(key)
-        if hit is not None and hit[0][0] is attn and hit[0][1] is enc and hit[0][2] is mask:
+        if hit is not None and hit[0][0] is attn and (cache_key is not None or (hit[0][1] is enc and hit[0][2] is mask)):
             return hit[1]
         B, Sk, _ = enc.shape
         k = attn.to_k(enc).view(B, Sk, H, -1)
@@ -165,9 +198,13 @@ class PikaH3AttnProcessor:
         if k.dtype != torch.bfloat16:
             k, v = k.to(torch.bfloat16), v.to(torch.bfloat16)
         kv = prepare_kv(k, v, **k_opts)
-        if len(self._cross_kv) >= 256:
-            self._cross_kv.pop(next(iter(self._cross_kv)))
-        self._cross_kv[key] = ((attn, enc, mask), kv)
+        self._cross_kv.pop(key, None)
+        # entries found by key do not need the tensors; entries found by tensor identity keep them alive
+        self._cross_kv[key] = ((attn, None, None) if cache_key is not None else (attn, enc, mask), kv)
+        total = sum(e[1].workspace.numel() for e in self._cross_kv.values())
+        while total > self.cross_kv_cache_bytes and len(self._cross_kv) > 1:
+            oldest = next(iter(self._cross_kv))
+            total -= self._cross_kv.pop(oldest)[1].workspace.numel()
         return kv
 
     def __call__(
@@ -186,6 +223,7 @@ class PikaH3AttnProcessor:
         gate: Optional[torch.Tensor] = None,
         gate_index: Optional[torch.Tensor] = None,
         residual: Optional[torch.Tensor] = None,
+        cross_kv_key: Optional[Hashable] = None,
     ) -> torch.Tensor:
         """``hidden_states [B, S, H*D]`` -> ``[B, S, H*D]``.
 
@@ -202,6 +240,10 @@ class PikaH3AttnProcessor:
         (patches/0001-h3-adaln-fp32.patch:34-40), and ``gate`` (bf16 ``[rows, C]``, gathered by ``gate_index``,
         int32 ``[S]``) and ``residual`` (``[B, S, C]``) make the result ``residual + gate * to_out(...)``.
         Without ``fused_projections`` those three arguments are rejected.
+
+        ``cross_kv_key`` (with ``cache_cross_kv``): the caller's name for the prompt whose text states this call
+        carries; prepared keys are then found by (module, key) instead of by tensor identity, see
+        :meth:`_prepared_cross_kv`.
         """
         if hidden_states.dim() != 3:
             raise ValueError(f"hidden_states must be [B, S, C], got {tuple(hidden_states.shape)}")
@@ -233,7 +275,7 @@ class PikaH3AttnProcessor:
             k_opts = dict(k_norm_weight=_norm_weight(kn, D, q.device), norm_eps=eps, fp8_qk=use_fp8)
             if attention_mask is not None:
                 k_opts.update(key_mask=attention_mask)
-            kv = self._prepared_cross_kv(attn, encoder_hidden_states, mask_given, k_opts, H)
+            kv = self._prepared_cross_kv(attn, encoder_hidden_states, mask_given, k_opts, H, cross_kv_key)
             out = attention_prepared(q, kv, q_norm_weight=_norm_weight(qn, D, q.device),
                                      softmax_scale=None if scale is None else float(scale))
             out = attn.to_out[0](out.view(B, S, H * D).to(hidden_states.dtype))

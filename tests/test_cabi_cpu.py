@@ -22,7 +22,7 @@ def test_header_symbols_are_exported(lib):
 
 
 def test_version_and_strerror(lib):
-    assert lib.pkh3_version() == 105
+    assert lib.pkh3_version() == 106
     assert lib.pkh3_strerror(0) == b"ok"
     assert b"128" in lib.pkh3_strerror(_lib.PKH3_EHEADDIM)
 

@@ -410,6 +410,59 @@ def test_processor_prepares_cross_attention_keys_once():
         cached(attn, x, encoder_hidden_states=enc)  # no mask: its own entry
         cached(attn, x, encoder_hidden_states=enc)
         assert calls["k"] - before == 1
+        # a prompt the caller names: new tensors in every step (a model that re-projects or re-concatenates its text
+        # states per forward hands over fresh ones) still find the prepared keys
+        cached.forget()
+        before = calls["k"]
+        for step in range(3):
+            got = cached(attn, x, encoder_hidden_states=enc.clone(), attention_mask=mask.clone(), cross_kv_key="prompt-1")
+        assert calls["k"] - before == 1
+        assert torch.equal(got, plain(attn, x, encoder_hidden_states=enc, attention_mask=mask))
+        # the K-side weights are part of the key: an in-place change prepares the keys again
+        attn.to_k.weight.mul_(1.25)
+        before = calls["k"]
+        got = cached(attn, x, encoder_hidden_states=enc.clone(), attention_mask=mask, cross_kv_key="prompt-1")
+        assert calls["k"] - before == 1
+        assert torch.equal(got, plain(attn, x, encoder_hidden_states=enc, attention_mask=mask))
+        # bounded by bytes, oldest entries first
+        small = pk.PikaH3AttnProcessor(cache_cross_kv=True, cross_kv_cache_bytes=1)
+        for name in range(3):
+            small(attn, x, encoder_hidden_states=enc, cross_kv_key=name)
+        assert len(small._cross_kv) == 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("scale", [0.05, 0.2])
+def test_processor_honours_the_modules_softmax_scale(scale):
+    """``attn.scale`` reaches the kernel: the processor against the oracle with the same scale, self-attention with
+    RoPE through the module projections and through the fused ones."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as O
+
+    torch.manual_seed(11)
+    H, hidden, S = 2, 256, 300
+    attn = _Attn(hidden, H).cuda().to(torch.bfloat16)
+    attn.scale = scale
+    x = torch.randn((1, S, hidden), device="cuda", dtype=torch.bfloat16)
+    pos = (torch.rand((S, 3), dtype=torch.float64) * 20).cuda()
+    with torch.no_grad():
+        q, k, v = (f(x).view(1, S, H, 128) for f in (attn.to_q, attn.to_k, attn.to_v))
+        ref = O.reference_layer(q.cpu(), k.cpu(), v.cpu(), q_norm_weight=attn.norm_q.weight.float().cpu(),
+                                k_norm_weight=attn.norm_k.weight.float().cpu(), rope_q=O.rope_tables(pos.cpu()),
+                                rope_mode=O.ROPE_INTERLEAVED, scale=scale)
+        other = O.reference_layer(q.cpu(), k.cpu(), v.cpu(), q_norm_weight=attn.norm_q.weight.float().cpu(),
+                                  k_norm_weight=attn.norm_k.weight.float().cpu(), rope_q=O.rope_tables(pos.cpu()),
+                                  rope_mode=O.ROPE_INTERLEAVED)
+        yref = attn.to_out[0](ref.to(torch.bfloat16).view(1, S, hidden).cuda())
+        yother = attn.to_out[0](other.to(torch.bfloat16).view(1, S, hidden).cuda())
+        for fused in (False, True):
+            y = pk.PikaH3AttnProcessor(fused_projections=fused)(attn, x, position_ids=pos)
+            err = float((y.float() - yref.float()).abs().max())
+            print(f"attn.scale={scale} fused={fused}: max_abs={err:.3e} (against 1/sqrt(D): "
+                  f"{float((y.float() - yother.float()).abs().max()):.3e})", flush=True)
+            assert err < 3e-2
+            # the scale matters at this size: the default-scale result is far outside the tolerance
+            assert float((y.float() - yother.float()).abs().max()) > 3 * err
 
 
 @pytest.mark.gpu

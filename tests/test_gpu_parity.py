@@ -23,7 +23,11 @@ def _rand(shape, gen, std=1.0):
 
 
 def _run_and_check(B, Sq, Sk, H, *, seed=0, norm=True, rope_mode=0, mask=None, std=1.0, min_cos=MIN_COS,
-                   max_abs=MAX_ABS, weight_random=False, weight_scale=1.0, bf16_operands=False):
+                   max_abs=MAX_ABS, weight_random=False, weight_scale=1.0, bf16_operands=False, fp8=False, scale=None,
+                   batch_pad=0):
+    """``fp8``: the fp8 QK^T path against the oracle's fake-quant emulation (cosine >= 0.995 by contract, held to
+    0.9995).  ``scale``: softmax scale other than 1/sqrt(D).  ``batch_pad``: extra elements between the batch entries
+    of q, k, v and the output, so the batch stride is not S*H*D."""
     import pika_h3_flex_amd as pk
 
     O = _oracle()
@@ -45,18 +49,33 @@ def _run_and_check(B, Sq, Sk, H, *, seed=0, norm=True, rope_mode=0, mask=None, s
         rope_q = O.rope_tables(posq)
         rope_k = O.rope_tables(posk)
     ref = O.reference_layer(q, k, v, q_norm_weight=qw, k_norm_weight=kw, rope_q=rope_q, rope_k=rope_k,
-                            rope_mode=rope_mode, key_mask=mask, bf16_operands=bf16_operands)
+                            rope_mode=rope_mode, key_mask=mask, bf16_operands=bf16_operands, fp8_qk=fp8, scale=scale)
     dev = "cuda"
     f32 = lambda t: None if t is None else t.to(torch.float32).contiguous().to(dev)
-    opts = dict(q_norm_weight=f32(qw), k_norm_weight=f32(kw), norm_eps=1e-6, rope_mode=rope_mode)
+    opts = dict(q_norm_weight=f32(qw), k_norm_weight=f32(kw), norm_eps=1e-6, rope_mode=rope_mode, fp8_qk=fp8,
+                softmax_scale=scale)
+    if fp8:
+        min_cos, max_abs = 0.9995, 2e-2
     if rope_mode:
         opts.update(rope_q=(f32(rope_q[0]), f32(rope_q[1])), rope_k=(f32(rope_k[0]), f32(rope_k[1])))
     if mask is not None:
         opts.update(key_mask=mask.to(dev))
     # calls with at most 16 key tiles normally take the short-key form of the kernel: check the long-key form
     # on the same inputs too, so both forms see every small case
+    def on_device(t):
+        """[B, S, H, D] on the card; with batch_pad as a view into a wider buffer, so the batch stride is S*H*D + pad"""
+        if not batch_pad:
+            return t.to(dev)
+        Bt, St = t.shape[0], t.shape[1]
+        buf = torch.full((Bt, St * H * D + batch_pad), float("nan"), dtype=torch.bfloat16, device=dev)
+        view = buf[:, :St * H * D].view(Bt, St, H, D)
+        view.copy_(t)
+        assert view.stride(0) == St * H * D + batch_pad
+        return view
+
     for long_form in (True, False):
-        out = pk.attention(q.to(dev), k.to(dev), v.to(dev), long_key_kernel=long_form, **opts)
+        o_buf = on_device(torch.zeros_like(q)) if batch_pad else None
+        out = pk.attention(on_device(q), on_device(k), on_device(v), long_key_kernel=long_form, out=o_buf, **opts)
         torch.cuda.synchronize()
         out = out.cpu()
         assert torch.isfinite(out.float()).all()
@@ -80,6 +99,73 @@ def test_ragged_lengths(S):
 @pytest.mark.parametrize("Sq,Sk", [(5, 300), (300, 5), (513, 129), (64, 4096)])
 def test_rectangular(Sq, Sk):
     _run_and_check(1, Sq, Sk, 3, seed=Sq + Sk)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("mode", [1, 2])
+@pytest.mark.parametrize("Sq,Sk", [(5, 300), (300, 5), (513, 129), (200, 2100)])
+def test_rectangular_with_rope_and_separate_tables(Sq, Sk, mode, fp8):
+    """Sq != Sk with rotation: the queries and the keys carry position grids of their own (distinct cos/sin tables);
+    both pairings, bf16 and fp8, both forms of the dense kernel (long_key_kernel on and off inside the helper)."""
+    _run_and_check(1, Sq, Sk, 2, seed=7 * Sq + Sk + mode, rope_mode=mode, weight_random=True, fp8=fp8)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("scale", [0.05, 0.2])
+def test_softmax_scale_other_than_default(scale, fp8):
+    """softmax_scale reaches the logits (bf16: folded into the Q operand; fp8: into the dequantisation factor).
+    0.2 with unit-weight QK-RMSNorm bounds the logits by 37 in log2 units: still the bounded-logit path."""
+    _run_and_check(1, 300, 420, 2, seed=int(scale * 100), rope_mode=1, scale=scale, fp8=fp8)
+
+
+def test_softmax_scale_on_the_running_max_path():
+    """scale 0.2 and norm weight x4: logit bound 148 in log2 units, far beyond the limit of the bounded-logit path."""
+    _run_and_check(1, 333, 333, 2, seed=21, rope_mode=2, scale=0.2, weight_scale=4.0, bf16_operands=True)
+
+
+def test_batch_stride_is_not_the_dense_one():
+    """B = 3 with 264 stray elements between batch entries of q, k, v and the output (batch stride != S*H*D)."""
+    _run_and_check(3, 130, 200, 2, seed=19, rope_mode=1, batch_pad=264)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_zero_rows_with_norm_eps_zero(fp8):
+    """norm_eps = 0 and an all-zero Q row and K row: the normalised rows are zeros (not 0 * inf), so the zero query
+    attends uniformly (its output is the mean of V) and the zero key gets logit 0 from every query; no NaN anywhere.
+    Checked against the oracle evaluated with zero rows replaced the same way."""
+    import pika_h3_flex_amd as pk
+
+    O = _oracle()
+    gen = torch.Generator().manual_seed(123)
+    B, Sq, Sk, H, D = 1, 150, 200, 2, 128
+    q, k, v = _rand((B, Sq, H, D), gen), _rand((B, Sk, H, D), gen), _rand((B, Sk, H, D), gen)
+    q[0, 17] = 0
+    q[0, 149, 1] = 0
+    k[0, 5] = 0
+    k[0, 199, 0] = 0
+    w = torch.ones(D)
+    pos_q = torch.rand((Sq, 3), generator=gen, dtype=torch.float64) * 20
+    pos_k = torch.rand((Sk, 3), generator=gen, dtype=torch.float64) * 20
+    tq, tk = O.rope_tables(pos_q), O.rope_tables(pos_k)
+    # the oracle's rms_norm gives 0 * inf = NaN on a zero row at eps = 0; the defined result is a zero row, which a
+    # vanishing eps reproduces exactly for the zero rows and to 1e-30 relative for the others
+    ref = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, norm_eps=1e-30, rope_q=tq, rope_k=tk, rope_mode=1,
+                            fp8_qk=fp8)
+    assert torch.isfinite(ref).all()
+    f32 = lambda t: t.float().contiguous().cuda()
+    for long_form in (False, True):
+        out = pk.attention(q.cuda(), k.cuda(), v.cuda(), q_norm_weight=w.cuda(), k_norm_weight=w.cuda(), norm_eps=0.0,
+                           rope_mode=1, rope_q=(f32(tq[0]), f32(tq[1])), rope_k=(f32(tk[0]), f32(tk[1])), fp8_qk=fp8,
+                           long_key_kernel=long_form)
+        torch.cuda.synchronize()
+        out = out.cpu()
+        assert torch.isfinite(out.float()).all()
+        err, cos = O.max_abs_and_cosine(out, ref)
+        print(f"eps=0 zero rows fp8={fp8} long_form={long_form}: max_abs={err:.3e} cos={cos:.7f}", flush=True)
+        assert err <= MAX_ABS and cos >= (0.9995 if fp8 else MIN_COS)
+        # the zero query row: uniform attention
+        mean_v = v.double().mean(dim=1)  # [B, H, D]
+        assert float((out[0, 17].double() - mean_v[0]).abs().max()) <= 1e-2
 
 
 def test_batch_and_heads():
@@ -178,12 +264,47 @@ def test_large_logits_with_key_mask():
     _run_and_check(2, 150, 333, 2, seed=78, mask=mask, weight_scale=4.0, bf16_operands=True)
 
 
-def test_bound_path_and_running_max_path_agree():
-    """Same inputs through both softmax formulations (the bound is forced off by PKH3_FORCE_ONLINE in a
-    fresh process in the benchmark scripts; here the two regimes are compared through the oracle only)."""
-    out_small, ref_small = _run_and_check(1, 500, 500, 2, seed=11, weight_scale=1.0)
-    out_big, ref_big = _run_and_check(1, 500, 500, 2, seed=11, weight_scale=4.0, bf16_operands=True)
+def test_both_softmax_forms_against_the_oracle_on_one_draw():
+    """One seed, two regimes: unit norm weights (logit bound 16.3: the bounded-logit softmax, no running maximum)
+    and weights x4 (bound 65: the running-max softmax).  Each is held to the oracle on its own inputs; the library
+    has no switch that forces one form onto the other's inputs, so the two forms are never run on identical logits
+    here -- `test_same_logits_through_both_softmax_forms` does that through the norm weights."""
+    out_small, _ = _run_and_check(1, 500, 500, 2, seed=11, weight_scale=1.0)
+    out_big, _ = _run_and_check(1, 500, 500, 2, seed=11, weight_scale=4.0, bf16_operands=True)
     assert not torch.equal(out_small, out_big)
+
+
+def test_same_logits_through_both_softmax_forms():
+    """The same logits through both softmax forms.  The kernel picks the form from the bound |q'| * max_j |k'_j| * scale
+    (bounded-logit form up to 48 in log2 units).  The queries here are zero in their last 8 head-dim elements, and one
+    extra key row is non-zero only there: its logit is exactly 0 for every query whatever its size, but its norm sets
+    max|k'|.  With the extra row all zero the bound is 16 and the bounded-logit form runs; with 300 in those 8
+    elements the bound is beyond 1000 and the running-max form runs -- on identical logits and values.  Both are held
+    to the oracle and must agree with each other to the rounding of the bf16 output."""
+    import pika_h3_flex_amd as pk
+
+    O = _oracle()
+    gen = torch.Generator().manual_seed(29)
+    B, S, H, D = 1, 400, 2, 128
+    q, k, v = _rand((B, S, H, D), gen), _rand((B, S + 1, H, D), gen), _rand((B, S + 1, H, D), gen)
+    q[..., 120:] = 0
+    k[:, S] = 0
+    k_big = k.clone()
+    k_big[:, S, :, 120:] = 300.0
+    w = torch.ones(D)
+    ref = O.reference_layer(q, k, v, q_norm_weight=w)
+    assert float((ref - O.reference_layer(q, k_big, v, q_norm_weight=w)).abs().max()) == 0.0  # the oracle sees no difference
+    for long_form in (False, True):
+        bounded = pk.attention(q.cuda(), k.cuda(), v.cuda(), q_norm_weight=w.cuda(), long_key_kernel=long_form)
+        running = pk.attention(q.cuda(), k_big.cuda(), v.cuda(), q_norm_weight=w.cuda(), long_key_kernel=long_form)
+        torch.cuda.synchronize()
+        e1, c1 = O.max_abs_and_cosine(bounded.cpu(), ref)
+        e2, c2 = O.max_abs_and_cosine(running.cpu(), ref)
+        e12, c12 = O.max_abs_and_cosine(bounded.cpu(), running.cpu())
+        print(f"long_form={long_form}: bounded vs oracle {e1:.3e}/{c1:.7f}; running-max vs oracle {e2:.3e}/{c2:.7f}; "
+              f"between them {e12:.3e}/{c12:.7f}", flush=True)
+        assert e1 <= MAX_ABS and c1 >= MIN_COS and e2 <= MAX_ABS and c2 >= MIN_COS
+        assert e12 <= 8e-3 and c12 >= 0.99999
 
 
 @pytest.mark.parametrize("variant", ["dense_rope_mask", "sparse_fp8", "long_dense_split_last_round"])

@@ -74,6 +74,28 @@ def test_adaln_modulate_matches_oracle(norm):
     assert AO.max_abs_and_cosine(row0, PO.adaln_modulate(x, shift=shift, scale=scale, norm=norm))[1] >= 0.99999
 
 
+def test_adaln_layer_norm_of_rows_with_a_large_common_offset():
+    """Rows whose mean is large against their spread (massive-activation channels): the variance must come from the
+    distances to the mean, not from E[x^2] - mean^2, which cancels in float32.  x = 0.25 * randn + 50 (bf16 grid step
+    0.25 at 50, so the spread is a few grid steps).  Also a constant row with eps = 0: zeros, not NaN."""
+    from oracle import attention_oracle as AO
+    from oracle import projection_oracle as PO
+    from pika_h3_flex_amd import projections as P
+
+    S, K = 200, 3072
+    x = (_r(S, K, seed=14) * 0.25 + 50.0).to(torch.bfloat16)
+    img = P.adaln_modulate(x.cuda(), norm="layer", eps=1e-6)
+    torch.cuda.synchronize()
+    got = _unpack(img, S, K).cpu()
+    ref = PO.adaln_modulate(x, norm="layer", eps=1e-6)
+    err, cos = AO.max_abs_and_cosine(got, ref)
+    print(f"adaln layer norm, offset rows: max_abs={err:.3e} cos={cos:.8f}", flush=True)
+    assert cos >= 0.99999 and float(((got.double() - ref).abs() / (ref.abs() + 1.0)).max()) <= 2.0 ** -8
+    const = torch.full((16, K), 3.0, dtype=torch.bfloat16)
+    out = _unpack(P.adaln_modulate(const.cuda(), norm="layer", eps=0.0), 16, K).cpu()
+    assert torch.count_nonzero(out) == 0 and torch.isfinite(out.float()).all()
+
+
 def _linear(n, k, seed, lora=True, bias=True):
     d = dict(weight=_r(n, k, seed=seed, std=k ** -0.5).to(torch.bfloat16))
     if bias:

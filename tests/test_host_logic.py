@@ -117,9 +117,20 @@ def test_key_padding_mask_forms():
     assert torch.equal(key_padding_mask(keep.to(torch.int64), 2, 5), keep)
     assert torch.equal(key_padding_mask(additive, 2, 5), keep)
     assert torch.equal(key_padding_mask(additive.to(torch.bfloat16)[:, None, None, :], 2, 5), keep)
-    assert torch.equal(key_padding_mask((additive * 0 - 10000.0 * (~keep))[:, None, :], 2, 5), keep)
+    assert torch.equal(key_padding_mask(torch.where(keep, 0.0, -10000.0)[:, None, :], 2, 5), keep)
     assert torch.equal(key_padding_mask(keep[:1], 2, 5), keep[:1].expand(2, 5))
     with pytest.raises(ValueError, match="queries or heads"):
         key_padding_mask(torch.zeros((2, 4, 7, 5)), 2, 5)
     with pytest.raises(ValueError, match="broadcast form"):
         key_padding_mask(keep, 2, 6)
+    # a float mask that is not additive {0, large negative}: a 0/1 keep-mask cast to float would keep every key,
+    # a soft bias would be collapsed to keep/drop -- both are refused
+    with pytest.raises(ValueError, match="additive"):
+        key_padding_mask(keep.to(torch.float32), 2, 5)
+    with pytest.raises(ValueError, match="additive"):
+        key_padding_mask(torch.full((2, 5), -0.5), 2, 5)
+    with pytest.raises(ValueError, match="additive"):
+        key_padding_mask(additive.to(torch.bfloat16) + 2.0, 2, 5)
+    with pytest.raises(ValueError, match="additive"):
+        key_padding_mask(torch.full((2, 5), float("nan")), 2, 5)
+    assert torch.equal(key_padding_mask(torch.where(keep, 0.0, -1e3), 2, 5), keep)

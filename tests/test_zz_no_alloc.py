@@ -82,3 +82,39 @@ def test_noalloc_rejects_calls_beyond_its_scratch():
     assert rc == _lib.PKH3_EWORKSPACE and b"scratch" in lib.pkh3_last_error()
     with pytest.raises(_lib.Pkh3Error):
         pk.attention(q, k, k, out=out, static_scratch=True)
+
+
+def test_noalloc_captured_into_a_hip_graph_replays_the_eager_bits():
+    """The entry point is meant for callers under HIP graph capture: after ``pkh3_noalloc_init`` (the look-ups that
+    are not stream operations) the call is captured, and every replay -- fresh inputs in the captured buffers, eager
+    work of the same entry point in between, which shares the built-in array -- gives the bits of an eager
+    ``pkh3_attn_fwd`` call on the same inputs."""
+    import pika_h3_flex_amd as pk
+
+    pk.ops.noalloc_init()
+    S, H = 700, 3
+    gen = torch.Generator().manual_seed(44)
+    rnd = lambda: torch.randn((1, S, H, D), generator=gen).to(torch.bfloat16).cuda()
+    q, k, v = rnd(), rnd(), rnd()
+    w = torch.ones(D, device="cuda")
+    pos = torch.rand((S, 3), generator=gen, dtype=torch.float64) * 20.0
+    opts = dict(q_norm_weight=w, k_norm_weight=w, rope_mode=1, rope_q=pk.rope_tables(pos.cuda()))
+    out = torch.empty_like(q)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        pk.attention(q, k, v, out=out, static_scratch=True, **opts)
+    for rep in range(3):
+        fresh = [rnd() for _ in range(3)]
+        eager = pk.attention(*fresh, **opts).clone()
+        # eager use of the shared array between the replays, with another shape
+        other = pk.attention(fresh[0][:, :200], fresh[1][:, :300], fresh[2][:, :300], static_scratch=True,
+                             q_norm_weight=w, k_norm_weight=w)
+        torch.cuda.synchronize()
+        for dst, src in zip((q, k, v), fresh):
+            dst.copy_(src)
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.isfinite(other.float()).all()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager call"
