@@ -10,6 +10,13 @@ attention kernel, inputs resident in HBM.
 Prints ONE JSON line: `value` = 4*Sq*Sk*D*H / step time in TFLOP/s; `roofline` prices the attention
 kernel alone (HIP events on its stream, inside the library) against the bf16 dense MFMA peak;
 `cpu_baseline` times torch's CPU scaled_dot_product_attention path on a declared query-row sample.
+
+The default run (workload 480p) then measures, outside the headline's timed region, the other
+workloads of the benchmark contract -- fp8 QK^T, block-sparse, block-sparse fp8, 768p, joint
+video+audio, text cross-attention, and the attention half of a 480p block through the library's
+projections -- and reports them under `config.other_workloads`, and the CPU-runnable configuration 1
+in full (torch CPU fp32 and bf16, and the library) under `cpu_baseline.config1`.  `--no-others` and
+any other `--workload` measure just the one workload.
 """
 import argparse
 import json
@@ -76,7 +83,7 @@ def _time_steps(step, steps, warmup):
     return mean, per[len(per) // 2], per[0]
 
 
-def bench_block(args, pk, workloads, dev) -> int:
+def bench_block(args, pk, workloads, dev) -> dict:
     """The attention half of one DiT block at 480p: AdaLN modulation -> to_q/to_k/to_v (+LoRA rank 128) -> attention ->
     to_out.0 (+LoRA) with gate and residual.  A "step" is that whole sequence through the library's projection GEMMs
     (K/V written by the GEMM epilogue in the attention kernel's layout); the same block with the projections and the
@@ -172,8 +179,119 @@ def bench_block(args, pk, workloads, dev) -> int:
                      "kernel_ms": round(ms_qkv, 4), "flops_per_launch": flops_qkv},
         "cpu_baseline": None,
     }
-    print(json.dumps(line))
-    return 0
+    return line
+
+
+ATTENTION_WORKLOADS = ("plumbing", "480p", "768p", "joint", "cross", "480p-sparse", "480p-sparse-fp8", "480p-fp8")
+# what the default run measures beside the headline (same process, after the headline's timed region)
+OTHER_WORKLOADS = ("480p-fp8", "480p-sparse", "480p-sparse-fp8", "768p", "joint", "cross", "480p-block")
+
+
+def algorithmic_bytes(B, Sq, Sk, H, D, fp8, density=1.0):
+    """Compulsory HBM bytes of one attention-kernel launch: Q read and O written once in bf16, the K' and V operand
+    images read once (K' one byte per element on the fp8 path).  Block-sparse calls still touch every K/V tile that
+    any row-block keeps, i.e. all of them at these densities."""
+    return float(B * H * D * (2 * Sq + 2 * Sq + (1 if fp8 else 2) * Sk + 2 * Sk))
+
+
+class AttentionCase:
+    """One attention workload set up on the device: inputs, options, output and workspace."""
+
+    def __init__(self, pk, workloads, name, seed, dev, inputs=None):
+        import torch
+
+        self.pk, self.name = pk, name
+        base = name.split("-")[0]
+        self.inp = inputs if inputs is not None else workloads.make(base, seed=seed, device=dev)
+        inp = self.inp
+        self.B, self.Sq, self.H, self.D = inp.q.shape
+        self.Sk = inp.k.shape[1]
+        self.ones = torch.ones(self.D, dtype=torch.float32, device=dev)
+        opts = dict(q_norm_weight=self.ones, k_norm_weight=self.ones, norm_eps=1e-6)
+        self.tabs = None
+        if inp.position_ids is not None:
+            self.tabs = pk.rope_tables(inp.position_ids)
+            opts.update(rope_mode=pk.ROPE_INTERLEAVED, rope_q=self.tabs)
+        if inp.key_mask is not None:
+            opts.update(key_mask=inp.key_mask)
+        self.density = 1.0
+        self.fp8 = name.endswith("fp8")
+        if "sparse" in name:
+            tm = pk.local_window_tile_map(self.Sq, inp.tokens_per_frame, window_frames=2, global_fraction=0.10, seed=seed)
+            self.density = float(tm.float().mean())
+            opts.update(block_mask=pk.BlockMask.from_dense(tm, device=dev))
+        if self.fp8:
+            opts.update(fp8_qk=True)
+        self.opts = opts
+        self.flops = inp.flops * self.density
+        self.out = torch.empty_like(inp.q)
+        args_ws, _keep = pk.ops.fill_args(inp.q, inp.k, inp.v, self.out, **opts)
+        self.ws = torch.empty(pk.ops.workspace_bytes(args_ws), dtype=torch.uint8, device=dev)
+
+    def step(self):
+        self.pk.attention(self.inp.q, self.inp.k, self.inp.v, out=self.out, workspace=self.ws, **self.opts)
+
+    def describe(self):
+        return (f"{self.name} attention layer: B={self.B}, H={self.H}, D={self.D}, Sq={self.Sq}, Sk={self.Sk}, "
+                f"QK-RMSNorm + 3-axis RoPE, non-causal" + (f", block-sparse density {self.density:.3f}" if self.density < 1 else ""))
+
+    def roofline(self, kernel_iters):
+        """The attention kernel alone (HIP events on its stream, inside the library) against its MFMA peak, beside
+        the bytes: algorithmic ones, and the profiled ones where a profile of this workload is committed."""
+        kernel_ms = self.pk.time_attention_kernel(self.inp.q, self.inp.k, self.inp.v, iters=kernel_iters, **self.opts)
+        achieved = self.flops / (kernel_ms * 1e-3) / 1e12
+        peak = PEAK_TFLOPS["fp8" if self.fp8 else "bf16"]
+        traffic, source = MEASURED_TRAFFIC.get(self.name, (None, None))
+        alg = algorithmic_bytes(self.B, self.Sq, self.Sk if self.inp.key_mask is None else int(self.inp.key_mask.sum()),
+                                self.H, self.D, self.fp8)
+        r = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+             "frac": round(achieved / peak, 4), "traffic": traffic, "traffic_source": source,
+             "algorithmic_bytes": alg, "traffic_over_algorithmic": None if traffic is None else round(traffic / alg, 2),
+             "kernel": "attn_fwd_kernel", "kernel_ms": round(kernel_ms, 4), "flops_per_launch": self.flops}
+        if traffic is not None:
+            # the other roof: bytes that crossed the L2 boundary per launch (profiled) over this run's kernel time
+            rate = traffic / (kernel_ms * 1e-3) / 1e9
+            r["traffic_rate_gbs"] = round(rate, 1)
+            r["traffic_frac_of_hbm_peak"] = round(rate / HBM_PEAK_GBS, 4)
+            r["binding_roof"] = "hbm" if rate / HBM_PEAK_GBS > achieved / peak else "mfma"
+        return r
+
+
+def other_workload_record(case, steps, warmup, kernel_iters):
+    ms, ms_median, ms_min = _time_steps(case.step, steps, warmup)
+    r = case.roofline(kernel_iters)
+    peak = r["peak"]
+    tflops = case.flops / (ms * 1e-3) / 1e12
+    return {"workload": case.describe(), "dtype": "fp8-e4m3 QK^T + bf16 PV" if case.fp8 else "bf16",
+            "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "ms_per_step_min": round(ms_min, 4),
+            "tflops": round(tflops, 2), "peak_tflops": peak, "frac": round(tflops / peak, 4),
+            "kernel_ms": r["kernel_ms"], "kernel_frac": r["frac"], "binding_roof": r.get("binding_roof", "mfma"),
+            "algorithmic_bytes": r["algorithmic_bytes"], "traffic": r["traffic"], "traffic_source": r["traffic_source"],
+            "traffic_ratio": r["traffic_over_algorithmic"], "traffic_frac_of_hbm_peak": r.get("traffic_frac_of_hbm_peak")}
+
+
+def config1_baselines(pk, workloads, dev, seed):
+    """The CPU-runnable configuration (B=1, H=4, S=1024, D=128, QK-RMSNorm, no mask) in full: torch CPU
+    scaled_dot_product_attention in fp32 and in bf16 on the host, and the library on the card."""
+    import torch
+
+    from oracle import cpu_sdpa
+
+    inp = workloads.make("plumbing", seed=seed, device=dev)
+    ones = torch.ones(128, dtype=torch.float32, device=dev)
+    flops = inp.flops
+    rec = {"workload": "B=1, H=4, S=1024, D=128, QK-RMSNorm (eps 1e-6, unit weight), no mask, non-causal; whole call", "flops": flops}
+    for name, dt in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        secs, threads = cpu_sdpa.time_cpu_baseline(inp.q, inp.k, inp.v, sample_rows=inp.q.shape[1], repeats=5,
+                                                   q_norm_weight=ones, k_norm_weight=ones, eps=1e-6, dtype=dt)
+        rec[f"cpu_{name}_ms"] = round(secs * 1e3, 3)
+        rec[f"cpu_{name}_tflops"] = round(flops / secs / 1e12, 4)
+        rec["cores"] = threads
+    out = torch.empty_like(inp.q)
+    ms, _, ms_min = _time_steps(lambda: pk.attention(inp.q, inp.k, inp.v, out=out, q_norm_weight=ones, k_norm_weight=ones), 50, 10)
+    rec["gpu_ms"] = round(ms, 4)
+    rec["gpu_tflops"] = round(flops / (ms * 1e-3) / 1e12, 2)
+    return rec
 
 
 def main() -> int:
@@ -181,10 +299,12 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="480p", choices=["plumbing", "480p", "768p", "joint", "cross", "480p-sparse", "480p-sparse-fp8", "480p-fp8", "480p-block"])
+    ap.add_argument("--workload", default="480p", choices=list(ATTENTION_WORKLOADS) + ["480p-block"])
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-rows", type=int, default=32768, help="query rows of the CPU baseline sample (0 = skip)")
     ap.add_argument("--kernel-iters", type=int, default=10)
+    ap.add_argument("--no-others", action="store_true",
+                    help="only the named workload: skip the other workloads and the config-1 baselines the default run adds")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy, a kernel of known traffic for scaling profiler byte counters")
     args = ap.parse_args()
@@ -208,36 +328,12 @@ def main() -> int:
     torch.cuda.set_device(0)
 
     if args.workload == "480p-block":
-        return bench_block(args, pk, workloads, dev)
+        print(json.dumps(bench_block(args, pk, workloads, dev)))
+        return 0
 
-    base = args.workload.split("-")[0]
-    inp = workloads.make(base, seed=args.seed, device=dev)
-    B, Sq, H, D = inp.q.shape
-    Sk = inp.k.shape[1]
-    ones = torch.ones(D, dtype=torch.float32, device=dev)
-    opts = dict(q_norm_weight=ones, k_norm_weight=ones, norm_eps=1e-6)
-    tabs = None
-    if inp.position_ids is not None:
-        tabs = pk.rope_tables(inp.position_ids)
-        opts.update(rope_mode=pk.ROPE_INTERLEAVED, rope_q=tabs)
-    if inp.key_mask is not None:
-        opts.update(key_mask=inp.key_mask)
-    density = 1.0
-    fp8 = args.workload.endswith("fp8")
-    if "sparse" in args.workload:
-        tm = pk.local_window_tile_map(Sq, inp.tokens_per_frame, window_frames=2, global_fraction=0.10, seed=args.seed)
-        density = float(tm.float().mean())
-        opts.update(block_mask=pk.BlockMask.from_dense(tm, device=dev))
-    if fp8:
-        opts.update(fp8_qk=True)
-    flops = inp.flops * density
-
-    out = torch.empty_like(inp.q)
-    args_ws, _keep = pk.ops.fill_args(inp.q, inp.k, inp.v, out, **opts)
-    ws = torch.empty(pk.ops.workspace_bytes(args_ws), dtype=torch.uint8, device=dev)
-
-    def step():
-        pk.attention(inp.q, inp.k, inp.v, out=out, workspace=ws, **opts)
+    case = AttentionCase(pk, workloads, args.workload, args.seed, dev)
+    inp, flops, fp8 = case.inp, case.flops, case.fp8
+    B, Sq, H, D, Sk = case.B, case.Sq, case.H, case.D, case.Sk
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
@@ -246,46 +342,47 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
     # the K timed steps, bracketed by synchronisation; per-step events (same stream) give median and minimum
-    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    t0 = time.perf_counter()
-    marks[0].record()
-    for i in range(args.steps):
-        step()
-        marks[i + 1].record()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
-    ms_median, ms_min = per_step[len(per_step) // 2], per_step[0]
+    ms_per_step, ms_median, ms_min = _time_steps(case.step, args.steps, args.warmup)
     value = flops / (ms_per_step * 1e-3) / 1e12
+    roofline = case.roofline(args.kernel_iters)
+    peak = roofline["peak"]
 
-    kernel_ms = pk.time_attention_kernel(inp.q, inp.k, inp.v, iters=args.kernel_iters, **opts)
-    achieved = flops / (kernel_ms * 1e-3) / 1e12
-    peak = PEAK_TFLOPS["fp8" if fp8 else "bf16"]
-    traffic = MEASURED_TRAFFIC.get(args.workload, (None, None))[0]
-    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload, (None, None))[0],
-                "traffic_source": MEASURED_TRAFFIC.get(args.workload, (None, None))[1], "kernel": "attn_fwd_kernel",
-                "kernel_ms": round(kernel_ms, 4), "flops_per_launch": flops}
-
-    if traffic is not None:
-        # the other roof: bytes that crossed the L2 boundary per launch (profiled) over this run's kernel time
-        rate = traffic / (kernel_ms * 1e-3) / 1e9
-        roofline["traffic_rate_gbs"] = round(rate, 1)
-        roofline["traffic_frac_of_hbm_peak"] = round(rate / HBM_PEAK_GBS, 4)
-        roofline["binding_roof"] = "hbm" if rate / HBM_PEAK_GBS > achieved / peak else "mfma"
+    others = None
+    config1 = None
+    if args.workload == "480p" and not args.no_others:
+        # Everything below runs after the headline's timed region, one workload at a time, each freed before the
+        # next: >= 5 warm-up and >= 10 timed layer calls each, the attention kernel alone timed beside them.
+        others = {}
+        o_steps, o_warm = max(10, args.steps // 2), max(5, args.warmup)
+        for name in OTHER_WORKLOADS:
+            if name == "480p-block":
+                b_args = argparse.Namespace(**{**vars(args), "steps": o_steps, "warmup": o_warm})
+                blk = bench_block(b_args, pk, workloads, dev)
+                others[name] = {"workload": blk["config"]["workload"], "dtype": "bf16", "steps": o_steps, "warmup": o_warm,
+                                "ms_per_step": blk["ms_per_step"], "tflops": blk["value"], "peak_tflops": PEAK_TFLOPS["bf16"],
+                                "frac": round(blk["value"] / PEAK_TFLOPS["bf16"], 4),
+                                "ms_per_step_with_torch_projections": blk["config"]["ms_per_step_with_torch_projections"],
+                                "ms_qkv_projection": blk["config"]["ms_qkv_projection"], "qkv_projection_frac": blk["roofline"]["frac"],
+                                "ms_out_projection": blk["config"]["ms_out_projection"], "ms_adaln_modulate": blk["config"]["ms_adaln_modulate"],
+                                "binding_roof": "mfma", "traffic": blk["roofline"]["traffic"], "traffic_source": blk["roofline"]["traffic_source"]}
+                continue
+            shares_inputs = name.split("-")[0] == "480p"
+            other = AttentionCase(pk, workloads, name, args.seed, dev, inputs=inp if shares_inputs else None)
+            others[name] = other_workload_record(other, o_steps, o_warm, args.kernel_iters)
+            del other
+            torch.cuda.empty_cache()
+        if args.cpu_rows > 0:
+            config1 = config1_baselines(pk, workloads, dev, args.seed)
 
     cpu = None
     if args.cpu_rows > 0:
         from oracle import cpu_sdpa
 
         rows = min(args.cpu_rows, Sq)
-        cpu_opts = dict(q_norm_weight=ones, k_norm_weight=ones, eps=1e-6, dtype=torch.float32)
-        if tabs is not None:
-            cpu_opts.update(rope_q=tabs)
+        cpu_opts = dict(q_norm_weight=case.ones, k_norm_weight=case.ones, eps=1e-6, dtype=torch.float32)
+        if case.tabs is not None:
+            cpu_opts.update(rope_q=case.tabs)
         if inp.key_mask is not None:
             cpu_opts.update(key_mask=inp.key_mask.cpu())
         secs, threads = cpu_sdpa.time_cpu_baseline(inp.q, inp.k, inp.v, sample_rows=rows, **cpu_opts)
@@ -296,19 +393,22 @@ def main() -> int:
                "cpu_model": cpu_model, "physical_cores": cpu_physical,
                "sample": f"torch CPU F.scaled_dot_product_attention fp32 (+RMSNorm, RoPE in torch) on the first {rows} of {Sq} "
                          f"query rows x all {Sk} keys x {H} heads, dense, one call of {secs:.2f} s; rate scales linearly in rows"}
+        if config1 is not None:
+            cpu["config1"] = config1
 
     line = {
         "metric": "attention TFLOP/s (4*Sq*Sk*D*H per layer call; prologue + attention kernel)",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8-e4m3 QK^T + bf16 PV" if fp8 else "bf16", "data": "synthetic",
-        "config": {"workload": f"{args.workload} attention layer: B={B}, H={H}, D={D}, Sq={Sq}, Sk={Sk}, "
-                               f"QK-RMSNorm + 3-axis RoPE, non-causal" + (f", block-sparse density {density:.3f}" if density < 1 else ""),
+        "config": {"workload": case.describe(),
                    "seed": args.seed, "pct_of_mfma_peak": round(100.0 * value / peak, 2),
                    "ms_per_step_median": round(ms_median, 4), "ms_per_step_min": round(ms_min, 4)},
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
+    if others is not None:
+        line["config"]["other_workloads"] = others
     print(json.dumps(line))
     return 0
 
