@@ -40,7 +40,7 @@
 extern "C" {
 #endif
 
-#define PKH3_VERSION 106
+#define PKH3_VERSION 107
 
 enum {
   PKH3_OK = 0,
@@ -77,6 +77,14 @@ enum {
                                  separate packing pass disappears.  B must be 1; o_sb, o_ss, o_sh are not read.  Rows
                                  of the buffer past ceil(Sq/32)*32 are left as they are (pkh3_out_proj never uses
                                  what it computes from them) */
+  PKH3_FLAG_FP8_POW2_SCALES = 1u << 4, /* with PKH3_FLAG_FP8_QK: another quantisation rule, for speed.  Every block
+                                 scale is the smallest power of two that is at least absmax / 448 (both formed in
+                                 float32), and Q is multiplied by softmax_scale * log2(e) before it is quantised instead
+                                 of its logits afterwards.  The matrix instruction then applies the scales itself and
+                                 the softmax needs no multiply per logit.  A K-side option too: pkh3_kv_prepare,
+                                 pkh3_qkv_proj and the calls on their keys must agree on it.  At most one binade of
+                                 the e4m3 range is given up; the error stays that of an e4m3 rounding (relative step
+                                 2^-4) */
   PKH3_FLAG_LONG_KEY_KERNEL = 1u << 1 /* dense calls with at most 16 key tiles (Sk <= 1024) normally run a
                                  short-key form of the kernel (small workgroups, three per CU); this flag
                                  selects the long-key form for them too.  Same results to the tolerance of the

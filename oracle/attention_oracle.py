@@ -30,6 +30,9 @@ Pinning status (tests/test_oracle.py):
   tile mask           pinned: equals dense attention with -inf on dropped tiles; full map == dense
   fp8_e4m3_round      pinned: exhaustive decode of all 256 codes + nearest-even brute force,
                       cross-checked against torch.float8_e4m3fn casts
+  pow2_ceil_f32       pinned: math.frexp over every float32 exponent (exact powers, one ulp above and
+                      below), and through fake_quant_fp8_blocks: scale in [absmax/448, 2*absmax/448),
+                      no saturation, error within half an e4m3 step of the scaled value
 Parity UNPINNED against the reference's real module (only an import of the pinned diffusers file
 could settle these; each is an explicit switch): RoPE pairing (interleaved vs half-split),
 frequency layout inside each axis slice and the axis order, use of raw float positions, norm
@@ -118,10 +121,23 @@ def fp8_e4m3_round_torch(x: torch.Tensor) -> torch.Tensor:
     return x.to(torch.float32).to(torch.float8_e4m3fn).to(torch.float64)
 
 
-def fake_quant_fp8_blocks(x: torch.Tensor, block: int = TILE) -> Tuple[torch.Tensor, torch.Tensor]:
+def pow2_ceil_f32(s: torch.Tensor) -> torch.Tensor:
+    """Smallest power of two >= ``s`` for positive normal float32 values, by the bits of the number: the exponent
+    field, plus one when any mantissa bit is set, clamped to the exponents an 8-bit E8M0 scale can name besides
+    its NaN code (2^-126 .. 2^127).  Pinned in tests/test_oracle.py against math.frexp over every exponent."""
+    bits = s.to(torch.float32).contiguous().view(torch.int32)
+    e = (bits >> 23) & 0xFF
+    e = e + ((bits & 0x7FFFFF) != 0).to(torch.int32)
+    e = e.clamp(1, 254)
+    return (e << 23).view(torch.float32)
+
+
+def fake_quant_fp8_blocks(x: torch.Tensor, block: int = TILE, pow2_scales: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """Quantise ``x [B, S, H, D]`` to e4m3 with one absmax scale per (batch, head, ``block`` rows)
     and return (dequantised float64 tensor, scales ``[B, H, ceil(S/block)]``).  The scale and the
-    division follow float32 arithmetic (scale = absmax / 448, value * (1 / scale)).  Runs on the
+    division follow float32 arithmetic (scale = absmax / 448, value * (1 / scale)).  With
+    ``pow2_scales`` the scale is the smallest power of two that is at least that float32 number (the
+    block-scale form of the OCP microscaling formats, whose scales are 8-bit exponents).  Runs on the
     device ``x`` lives on: NumPy rounding on the host, torch's e4m3 cast elsewhere."""
     B, S, H, D = x.shape
     nb = (S + block - 1) // block
@@ -131,6 +147,8 @@ def fake_quant_fp8_blocks(x: torch.Tensor, block: int = TILE) -> Tuple[torch.Ten
     blk = x32.view(B, nb, block, H, D)
     amax = blk.abs().amax(dim=(2, 4))                                   # [B, nb, H]
     sc = torch.where(amax > 0, amax * np.float32(1.0 / FP8_MAX), torch.ones_like(amax))
+    if pow2_scales:
+        sc = torch.where(amax > 0, pow2_ceil_f32(sc), sc)
     inv = (torch.ones_like(sc) / sc)[:, :, None, :, None]
     scaled = blk * inv                                                  # float32, |.| <= 448
     if dev.type == "cpu":
@@ -197,10 +215,13 @@ def attention(
 def reference_layer(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, q_norm_weight=None, k_norm_weight=None,
     norm_eps: float = 1e-6, rope_q=None, rope_k=None, rope_mode: int = ROPE_NONE, key_mask=None,
-    tile_map=None, fp8_qk: bool = False, scale: Optional[float] = None, q_rows=None, bf16_operands: bool = False,
+    tile_map=None, fp8_qk=False, scale: Optional[float] = None, q_rows=None, bf16_operands: bool = False,
 ) -> torch.Tensor:
     """The whole path on ``[B, S, H, D]`` inputs: QK-RMSNorm -> RoPE -> (fp8 fake-quant of Q, K) ->
     masked softmax attention, float64.  A ``None`` norm weight means no norm on that side.
+    ``fp8_qk``: False, True (absmax / 448 block scales) or ``"pow2"``: power-of-two block scales, and the
+    normed/rotated Q is multiplied by ``scale * log2(e)`` (in float32) BEFORE it is quantised -- the form in
+    which a matrix unit with built-in block scaling needs no multiply per logit afterwards.
     ``bf16_operands`` rounds the normed/rotated K, and the normed/rotated Q times
     ``scale * log2(e)`` (the factor a log2-domain kernel carries in its Q operand), to bf16 first: the
     precision a bf16 matrix unit sees.  Used where logits are so large that this rounding alone
@@ -219,7 +240,13 @@ def reference_layer(
         cq = (float(scale) if scale is not None else q.shape[-1] ** -0.5) * math.log2(math.e)
         qf = (qf * cq).to(torch.bfloat16).to(torch.float64) / cq
         kf = kf.to(torch.bfloat16).to(torch.float64)
-    if fp8_qk:
+    if fp8_qk == "pow2":
+        sm = np.float32(float(scale) if scale is not None else q.shape[-1] ** -0.5)
+        cq = float(sm * np.float32(1.4426950408889634))        # the factor as the kernel forms it, in float32
+        qf, _ = fake_quant_fp8_blocks(qf.to(torch.float32) * cq, pow2_scales=True)
+        qf = qf / cq
+        kf, _ = fake_quant_fp8_blocks(kf, pow2_scales=True)
+    elif fp8_qk:
         qf, _ = fake_quant_fp8_blocks(qf)
         kf, _ = fake_quant_fp8_blocks(kf)
     return attention(qf, kf, v, scale=scale, key_mask=key_mask, tile_map=tile_map, q_rows=q_rows)

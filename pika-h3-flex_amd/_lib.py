@@ -27,6 +27,7 @@ FLAG_FP8_QK = 1
 FLAG_LONG_KEY_KERNEL = 2
 FLAG_KV_PREPARED = 4
 FLAG_O_IMAGES = 8
+FLAG_FP8_POW2_SCALES = 16
 NORM_NONE, NORM_LAYER, NORM_RMS = 0, 1, 2
 LORA_RANK = 128  # PKH3_LORA_RANK
 NOALLOC_SCRATCH_BYTES = 64 << 20  # PKH3_NOALLOC_SCRATCH_BYTES

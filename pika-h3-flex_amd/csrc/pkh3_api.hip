@@ -53,8 +53,11 @@ int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = tru
   // workgroup counts and tile indices are 32-bit: at most 2^30 blocks of 32 queries per call
   if ((int64_t)a->B * a->H * ((a->Sq + 31) / 32) > (1ll << 30))
     return fail(PKH3_ESHAPE, "B * H * ceil(Sq / 32) must be <= 2^30");
-  if (a->flags & ~(uint32_t)(PKH3_FLAG_FP8_QK | PKH3_FLAG_LONG_KEY_KERNEL | PKH3_FLAG_KV_PREPARED | PKH3_FLAG_O_IMAGES))
+  if (a->flags & ~(uint32_t)(PKH3_FLAG_FP8_QK | PKH3_FLAG_LONG_KEY_KERNEL | PKH3_FLAG_KV_PREPARED | PKH3_FLAG_O_IMAGES |
+                             PKH3_FLAG_FP8_POW2_SCALES))
     return fail(PKH3_EARG, "unknown flag bits 0x%x", a->flags);
+  if ((a->flags & PKH3_FLAG_FP8_POW2_SCALES) && !(a->flags & PKH3_FLAG_FP8_QK))
+    return fail(PKH3_EARG, "PKH3_FLAG_FP8_POW2_SCALES is an option of PKH3_FLAG_FP8_QK");
   if ((a->flags & PKH3_FLAG_O_IMAGES) && a->B != 1)
     return fail(PKH3_EUNSUPPORTED, "output as operand images (PKH3_FLAG_O_IMAGES) means one document: B = 1");
   if (a->rope_mode < PKH3_ROPE_NONE || a->rope_mode > PKH3_ROPE_HALF) return fail(PKH3_EARG, "bad rope_mode %d", a->rope_mode);
@@ -143,6 +146,7 @@ void build(const pkh3_attn_args* a, void* workspace, Launch& L) {
   k.gather_idx = L.idx; k.row_cnt = L.cnt;
   k.out = ws + L.w.kv_off; k.out_bh_stride = (int64_t)L.w.nKt * L.w.kvTileBytes; k.out_blk_stride = L.w.kvTileBytes;
   k.scale_out = fp8 ? (float*)(ws + L.w.kscale_off) : nullptr; k.fp8 = fp8;
+  k.fp8_pow2 = (a->flags & PKH3_FLAG_FP8_POW2_SCALES) ? 1 : 0;
   k.norm_max = (unsigned*)(ws + L.w.kmax_off);
 
   VPrologueParams& v = L.vp;
@@ -170,7 +174,7 @@ void build(const pkh3_attn_args* a, void* workspace, Launch& L) {
   f.plan = a->blk_row_ptr ? (const int*)(ws + L.w.plan_off) : nullptr;
   f.plan_cnt = a->blk_row_ptr ? (const int*)(ws + L.w.plan_cnt_off) : nullptr;
   f.plan_stride = kSparseLists * L.w.nKt;
-  f.kscale = k.scale_out; f.fp8 = fp8; f.long_key_kernel = (a->flags & PKH3_FLAG_LONG_KEY_KERNEL) ? 1 : 0;
+  f.kscale = k.scale_out; f.fp8 = fp8; f.fp8_pow2 = k.fp8_pow2; f.long_key_kernel = (a->flags & PKH3_FLAG_LONG_KEY_KERNEL) ? 1 : 0;
   f.kmax = (const float*)(ws + L.w.kmax_off);
 }
 
@@ -518,7 +522,7 @@ int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream)
     GemmTarget& k = g.tg[1];
     k.epi = kEpiKImg; k.out = L.kp.out; k.out_head_stride = L.kp.out_bh_stride; k.out_blk_stride = L.kp.out_blk_stride;
     k.norm_w = a->k_norm_w; k.norm_eps = a->norm_eps; k.rope_mode = a->rope_mode; k.cos_t = a->k_rope_cos; k.sin_t = a->k_rope_sin;
-    k.norm_max = L.kp.norm_max; k.fp8 = fp8; k.scale_out = L.kp.scale_out; k.scale_head_stride = L.w.nKt;
+    k.norm_max = L.kp.norm_max; k.fp8 = fp8; k.fp8_pow2 = L.kp.fp8_pow2; k.scale_out = L.kp.scale_out; k.scale_head_stride = L.w.nKt;
     GemmTarget& v = g.tg[2];
     v.epi = kEpiVImg; v.out = L.vp.out; v.out_head_stride = L.vp.out_bh_stride; v.out_blk_stride = L.vp.out_tile_stride;
   }

@@ -100,19 +100,25 @@ struct WaveState {
   f32x4 o[8][2];                        // O^T accumulators (db, qb): head-dim rows 16*db + 4*g + i
   bf16x8 vf[8];                         // V images of the first 32 keys, fetched while QK^T finishes
   float m[2], l[2];                     // per query block: running row max (scaled, log2 domain), this lane group's row sum
+  int qe;                               // fp8 with power-of-two scales: exponent byte (E8M0) of the Q block's scale
 };
 
 #define PKH3_MFMA16(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, B, C, 0, 0, 0)
 // format codes 0/0 = e4m3 x e4m3; scale operands 0 select the unscaled form of the instruction
 #define PKH3_MFMA16_F8(A, B, C) __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C, 0, 0, 0, 0, 0, 0)
+// the scaled form: the product is multiplied by 2^(EA - 127) * 2^(EB - 127), EA / EB = byte 0 of each lane's scale
+// operand (every lane passes the same exponents: one scale per 64-row block, not per 32 elements)
+#define PKH3_MFMA16_F8S(A, B, C, EA, EB) __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C, 0, 0, 0, EA, 0, EB)
 
 // S^T = K' Q'^T for the 64 keys of one tile: image i of the K tile is (half, ks, kb2) = (i >> 3, (i >> 1) & 3, i & 1)
 // and feeds the two query blocks, so four accumulators rotate inside each half.  LDS reads run 8 images ahead of
 // the MFMAs that consume them; the tail of the MFMA chain covers the first V image reads.
 // LEAN (three waves per SIMD, 168 VGPRs): the reads run only 4 images ahead and V is left to the P.V loop.
 // AHEAD: images the LEAN reads run ahead (the copies of the loop that run once per workgroup take 2 and fit the registers)
-template <bool FP8, bool LEAN, int AHEAD = 4>
-__device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane) {
+// POW2 (fp8): the block scales are powers of two and go into the MFMA as its scale operands (`ke`: exponent byte of
+// this K tile's scale), so S^T leaves the MFMA dequantised.
+template <bool FP8, bool LEAN, int AHEAD = 4, bool POW2 = false>
+__device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane, int ke = 0) {
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   if constexpr (!FP8 && LEAN) {
     bf16x8 kf[16];
@@ -160,7 +166,8 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
       const i32x4 a0 = kc[2 * kb], a1 = kc[2 * kb + 1];
       const i32x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) w.s[kb][qb] = PKH3_MFMA16_F8(a, w.q8[qb], zero);
+      for (int qb = 0; qb < 2; ++qb)
+        w.s[kb][qb] = POW2 ? PKH3_MFMA16_F8S(a, w.q8[qb], zero, ke, w.qe) : PKH3_MFMA16_F8(a, w.q8[qb], zero);
       // the MFMA chain covers the first V image reads: 8 images, or 4 where registers are short (LEAN)
       if constexpr (LEAN) {
         w.vf[kb] = *(const bf16x8*)(vbuf + (kb * 64 + lane) * 16);
@@ -172,12 +179,13 @@ __device__ __forceinline__ void qk_tile(WaveState<FP8>& w, const char* kbuf, con
   }
 }
 
-// exp2 of one logit.  bf16 path: Q' already carries softmax_scale * log2(e), so S^T is in the log2 domain and
-// `c` is unused; fp8 path: `c` carries that factor times the dequantisation scales.  STATIC: the logits are
-// bounded in magnitude (see kStaticMaxLimit), so no maximum is subtracted at all.
-template <bool FP8, bool STATIC>
+// exp2 of one logit.  bf16 path, and fp8 with power-of-two scales: Q' already carries softmax_scale * log2(e) (and the
+// MFMA applied the scales), so S^T is in the log2 domain and `c` is unused; fp8 with absmax scales (MUL): `c` carries
+// that factor times the dequantisation scales.  STATIC: the logits are bounded in magnitude (see kStaticMaxLimit), so
+// no maximum is subtracted at all.
+template <bool MUL, bool STATIC>
 __device__ __forceinline__ float softmax_numerator(float s, float c, float m) {
-  if constexpr (FP8) return __builtin_amdgcn_exp2f(STATIC ? s * c : fmaf(s, c, -m));
+  if constexpr (MUL) return __builtin_amdgcn_exp2f(STATIC ? s * c : fmaf(s, c, -m));
   else return __builtin_amdgcn_exp2f(STATIC ? s : s - m);
 }
 
@@ -188,8 +196,9 @@ __device__ __forceinline__ float softmax_numerator(float s, float c, float m) {
 // STATIC: w.m is not used: every logit is bounded (|q_i| * max_j |k_j| * c), small enough that exp2(logit) is a
 // normal number; the running max, its exchange across the lane groups and the O^T rescale are then not needed at
 // all, and the numerators of the first 32 keys do not wait for the second half of S^T.
-template <bool FP8, bool STATIC, bool MASKED, int NKB>
+template <bool FP8, bool STATIC, bool MASKED, int NKB, bool POW2 = false>
 __device__ __forceinline__ void softmax_blocks(WaveState<FP8>& w, bf16x8 (&pf)[NKB / 2][2], float c, int lim, int lane) {
+  constexpr bool MUL = FP8 && !POW2;  // the logits still need their dequantisation scales
   const int g = lane >> 4;
   if (MASKED) {
 #pragma unroll
@@ -210,7 +219,7 @@ __device__ __forceinline__ void softmax_blocks(WaveState<FP8>& w, bf16x8 (&pf)[N
       for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mx = fmaxf(mx, w.s[kb][qb][i]);
-      mx = max_across_groups(mx) * (FP8 ? c : 1.0f);
+      mx = max_across_groups(mx) * (MUL ? c : 1.0f);
       m_new[qb] = (mx > w.m[qb] + kRescaleSlack) ? mx : w.m[qb];
       alpha[qb] = __builtin_amdgcn_exp2f(w.m[qb] - m_new[qb]);
       w.m[qb] = m_new[qb];
@@ -233,7 +242,7 @@ __device__ __forceinline__ void softmax_blocks(WaveState<FP8>& w, bf16x8 (&pf)[N
       bf16x8 pk;
 #pragma unroll
       for (int j = 0; j < 8; ++j)
-        pk[j] = (__bf16)softmax_numerator<FP8, STATIC>(w.s[2 * half + (j >> 2)][qb][j & 3], c, m_new[qb]);
+        pk[j] = (__bf16)softmax_numerator<MUL, STATIC>(w.s[2 * half + (j >> 2)][qb][j & 3], c, m_new[qb]);
       // row sum over the bf16-rounded values, the same numbers the P.V MFMA consumes
 #pragma unroll
       for (int j = 0; j < 8; j += 2) {
@@ -249,10 +258,10 @@ __device__ __forceinline__ void softmax_blocks(WaveState<FP8>& w, bf16x8 (&pf)[N
 // Softmax of w.s, then O^T += V^T P^T for one tile: V image i is (half, db) = (i >> 3, i & 7) and feeds the two
 // query blocks, sixteen accumulators in rotation.  `c` = softmax scale * log2(e) (times the fp8 dequantisation
 // scales of this tile); `lim` = keys of this tile that exist (only read when MASKED).
-template <bool FP8, bool STATIC, bool LEAN, bool MASKED>
+template <bool FP8, bool STATIC, bool LEAN, bool MASKED, bool POW2 = false>
 __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* vbuf, float c, int lim, int lane) {
   bf16x8 pf[2][2];
-  softmax_blocks<FP8, STATIC, MASKED, 4>(w, pf, c, lim, lane);
+  softmax_blocks<FP8, STATIC, MASKED, 4, POW2>(w, pf, c, lim, lane);
   if constexpr (LEAN) {
     bf16x8 vg[16];
 #pragma unroll
@@ -278,8 +287,8 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
 // S^T (32 keys x 32 queries) into w.s[0..1]; kbuf/vbuf point at this half's K images (8 bf16 / 4 fp8 chunks)
 // and V images (8).
 // LEAN (three waves per SIMD): the K reads run 4 images ahead and only the fp8 path prefetches V (4 images).
-template <bool FP8, bool LEAN = false>
-__device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane) {
+template <bool FP8, bool LEAN = false, bool POW2 = false>
+__device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, const char* vbuf, int lane, int ke = 0) {
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   if constexpr (!FP8 && LEAN) {
     bf16x8 kf[8];
@@ -310,7 +319,8 @@ __device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, con
       const i32x4 a0 = kc[2 * kb], a1 = kc[2 * kb + 1];
       const i32x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) w.s[kb][qb] = PKH3_MFMA16_F8(a, w.q8[qb], zero);
+      for (int qb = 0; qb < 2; ++qb)
+        w.s[kb][qb] = POW2 ? PKH3_MFMA16_F8S(a, w.q8[qb], zero, ke, w.qe) : PKH3_MFMA16_F8(a, w.q8[qb], zero);
 #pragma unroll
       for (int i = 0; i < (LEAN ? 2 : 4); ++i) {
         const int v = (LEAN ? 2 : 4) * kb + i;
@@ -324,12 +334,12 @@ __device__ __forceinline__ void qk_half(WaveState<FP8>& w, const char* kbuf, con
 // `lim` = keys of this half that exist (<= 0: none; only read when < 32).
 // LEAN: the V images (beyond the 4 the fp8 path prefetched) are read here, 4 ahead of their MFMAs, from vbuf.
 // FULL: the caller guarantees lim == 32, no masking code at all.
-template <bool FP8, bool STATIC, bool LEAN = false, bool FULL = false>
+template <bool FP8, bool STATIC, bool LEAN = false, bool FULL = false, bool POW2 = false>
 __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int lim, int lane, const char* vbuf = nullptr) {
   bf16x8 pf[1][2];
   // the running-max form always takes the masking copy (two copies of it do not fit the registers of some variants)
-  if (!FULL && (!STATIC || lim < 32)) softmax_blocks<FP8, STATIC, true, 2>(w, pf, c, lim, lane);
-  else softmax_blocks<FP8, STATIC, false, 2>(w, pf, c, lim, lane);
+  if (!FULL && (!STATIC || lim < 32)) softmax_blocks<FP8, STATIC, true, 2, POW2>(w, pf, c, lim, lane);
+  else softmax_blocks<FP8, STATIC, false, 2, POW2>(w, pf, c, lim, lane);
   if constexpr (LEAN) {
     bf16x8 vg[8];
 #pragma unroll
@@ -356,9 +366,12 @@ __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int 
 // 128 queries instead of 384 and its three groups of 4 waves walk one third of the keys each (half tiles, a ring
 // per group), then add their partial results up through LDS.  Such a workgroup lasts a third as long, so the
 // CUs that would idle through a whole round of whole workgroups idle through a third of one.
-template <bool FP8, bool SPARSE, int WAVES, bool SPLIT = false>
+// POW2 (fp8 only): power-of-two block scales, applied by the scaled MFMA; softmax_scale * log2(e) rides in Q' before
+// it is quantised, so the softmax has no multiply left (the instruction count of the bf16 form).
+template <bool FP8, bool SPARSE, int WAVES, bool SPLIT = false, bool POW2 = false>
 __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWaves ? 3 : 1)) void attn_fwd_kernel(FwdParams p) {
   static_assert(!SPARSE || WAVES == kSparseWaves, "block-sparse layout: a wave pair per row-block of the plan");
+  static_assert(FP8 || !POW2, "power-of-two scales belong to the fp8 form");
   constexpr bool SHORT = !SPARSE && WAVES == kShortWaves;
   constexpr bool LEAN = !SPARSE;                        // dense long-key form: three waves per SIMD, lean read-ahead
   // whole-tile ring depth: three tiles, except where two workgroups share the CU's LDS and a bf16 tile is 32 KiB
@@ -508,13 +521,19 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
       // one absmax scale per 64-query block = this wave and its neighbour (wave ^ 1)
       __shared__ float q_amax[WAVES];
       float amax = 0.f;
+      if constexpr (POW2) {
+        // softmax_scale * log2(e) goes into Q' before the quantisation, as in the bf16 form
+#pragma unroll
+        for (int i = 0; i < 64; ++i) x[i] *= p.c;
+      }
 #pragma unroll
       for (int i = 0; i < 64; ++i) amax = fmaxf(amax, fabsf(x[i]));
       amax = wave_max(amax);
       if (lane == 0) q_amax[wave] = amax;
       __syncthreads();
       amax = fmaxf(amax, q_amax[wave ^ 1]);
-      qscale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
+      qscale = fp8_block_scale(amax, POW2);
+      w.qe = e8m0_of(qscale);
       const float inv = 1.0f / qscale;
       i32x4 qold[4];
 #pragma unroll
@@ -549,7 +568,7 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
       for (int i = 0; i < 4; ++i) w.o[db][qb][i] = 0.f;
   w.m[0] = w.m[1] = -INFINITY;
   w.l[0] = w.l[1] = 0.f;
-  const float c = p.c * qscale;
+  const float c = POW2 ? 1.0f : p.c * qscale;  // what the softmax still multiplies the logits by (fp8 absmax form only)
   const float* kscale = FP8 ? p.kscale + (int64_t)bh * p.nKt : nullptr;
   const int tail = sk & (kTileKeys - 1);  // keys in the last tile when it is partial
 
@@ -559,7 +578,7 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   bool static_max = false;
   if (HALFMODE ? n_half > 0 : nt > 0) {
     // margins: K' is rounded to bf16 (fp8: to e4m3, relative step 2^-4) after its norm was taken
-    const float bound = sqrtf(qn2) * uniform_load(p.kmax, bh) * (FP8 ? p.c * 1.08f : 1.01f);
+    const float bound = sqrtf(qn2) * uniform_load(p.kmax, bh) * (FP8 ? (POW2 ? 1.08f : p.c * 1.08f) : 1.01f);
     static_max = __all(bound <= kStaticMaxLimit);
   }
 
@@ -576,14 +595,15 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     __syncthreads();                                                                                    \
     const char* kbuf = lds[slot];                                                                       \
     const int tile = entry(i);                                                                          \
-    qk_tile<FP8, LEAN, (MASKED) ? 2 : 4>(w, kbuf, kbuf + kKBytes, lane);                                \
+    const float ks = FP8 ? uniform_load(kscale, tile) : 1.0f;                                           \
+    qk_tile<FP8, LEAN, (MASKED) ? 2 : 4, POW2>(w, kbuf, kbuf + kKBytes, lane, e8m0_of(ks));             \
     /* the copies of the tile two ahead are issued under the MFMAs of S^T, not in front of them: right */ \
     /* after the barrier their scalar address chain would run in every wave at once with the pipe idle */ \
     if (i + kAhead < nt) dma(entry(i + kAhead), slot_prev);                                             \
     slot_prev = slot;                                                                                   \
     slot = slot == kRingT - 1 ? 0 : slot + 1;                                                           \
-    const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
-    softmax_pv_tile<FP8, STATIC, LEAN, MASKED>(w, kbuf + kKBytes, ct, tail, lane);                      \
+    const float ct = (FP8 && !POW2) ? c * ks : c;                                                       \
+    softmax_pv_tile<FP8, STATIC, LEAN, MASKED, POW2>(w, kbuf + kKBytes, ct, tail, lane);                \
   }
   // Half-tile loop.  Every wave runs the same number of iterations (the longest group's), so the barriers match.
   // A group's leading full halves take the copy of the code without masking; what is left -- at most the one
@@ -595,14 +615,15 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     const char* hbuf = ring + slot * kHalfBytes;                                                        \
     const int half = h_begin + i;                                                                       \
     const bool live = FULL || i < n_mine;                                                               \
-    if (live) qk_half<FP8, true>(w, hbuf, hbuf + kKHalfB, lane);                                        \
+    const float ks = (FP8 && live) ? uniform_load(kscale, half >> 1) : 1.0f;                            \
+    if (live) qk_half<FP8, true, POW2>(w, hbuf, hbuf + kKHalfB, lane, e8m0_of(ks));                     \
     /* copies of the half two ahead: under the MFMAs of S^T (see the whole-tile loop) */               \
     if (i + 2 < n_mine) dma_short(h_begin + i + 2, slot_prev);                                          \
     slot_prev = slot;                                                                                   \
     slot = slot == kRing - 1 ? 0 : slot + 1;                                                            \
     if (live) {                                                                                         \
-      const float ct = FP8 ? c * uniform_load(kscale, half >> 1) : c;                                   \
-      softmax_pv_half<FP8, STATIC, true, FULL>(w, ct, sk - 32 * half, lane, hbuf + kKHalfB);            \
+      const float ct = (FP8 && !POW2) ? c * ks : c;                                                     \
+      softmax_pv_half<FP8, STATIC, true, FULL, POW2>(w, ct, sk - 32 * half, lane, hbuf + kKHalfB);      \
     }                                                                                                   \
   }
   if constexpr (HALFMODE) {
@@ -716,12 +737,13 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     if (it >= 2 * n_mine) continue; /* wave-uniform: this row-block has run out of tiles (and of copies) */ \
     const int tile = uniform_load(mine, it >> 1);                                                       \
     /* the running-max copy needs registers for the rescale: it takes the lean read-ahead (4 images) */ \
-    qk_half<FP8, !STATIC>(w, hbuf, hbuf + kKHalf, lane);                                                \
+    const float ks = FP8 ? uniform_load(kscale, tile) : 1.0f;                                           \
+    qk_half<FP8, !STATIC, POW2>(w, hbuf, hbuf + kKHalf, lane, e8m0_of(ks));                             \
     /* copies of the next half tile of this row-block: under the MFMAs of S^T (see the whole-tile loop) */ \
     if (it + kStages2 - 1 < 2 * n_mine) dma_half(it + kStages2 - 1, st2_write);                         \
-    const float ct = FP8 ? c * uniform_load(kscale, tile) : c;                                          \
+    const float ct = (FP8 && !POW2) ? c * ks : c;                                                       \
     const int lim = (tail && tile == nkt - 1) ? tail - 32 * (it & 1) : 32;                              \
-    softmax_pv_half<FP8, STATIC, !STATIC>(w, ct, lim, lane, hbuf + kKHalf);                             \
+    softmax_pv_half<FP8, STATIC, !STATIC, false, POW2>(w, ct, lim, lane, hbuf + kKHalf);                \
   }
     if (static_max) {
       PKH3_HALF_LOOP(true)
@@ -790,19 +812,19 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   }
 }
 
-template <bool FP8, bool SPARSE, int WAVES, bool SPLIT = false>
+template <bool FP8, bool POW2, bool SPARSE, int WAVES, bool SPLIT = false>
 static void launch_variant(FwdParams p, int unit0, int units, hipStream_t st) {
   p.unit0 = unit0;
   p.units = units;
-  hipLaunchKernelGGL((attn_fwd_kernel<FP8, SPARSE, WAVES, SPLIT>), dim3((units + 7) / 8 * 8), dim3(64 * WAVES), 0, st, p);
+  hipLaunchKernelGGL((attn_fwd_kernel<FP8, SPARSE, WAVES, SPLIT, POW2>), dim3((units + 7) / 8 * 8), dim3(64 * WAVES), 0, st, p);
 }
 
-template <bool FP8>
+template <bool FP8, bool POW2 = false>
 static void launch_fp(const FwdParams& p, int cus, hipStream_t st) {
   const int nQ32 = p.nQ64 * 2;
   auto units = [&](int blocks) { return p.B * p.H * ((nQ32 + blocks - 1) / blocks); };
-  if (p.plan) return launch_variant<FP8, true, kSparseWaves>(p, 0, units(kSparseWaves), st);
-  if (p.nKt <= kShortMaxTiles && !p.long_key_kernel) return launch_variant<FP8, false, kShortWaves>(p, 0, units(kShortWaves), st);
+  if (p.plan) return launch_variant<FP8, POW2, true, kSparseWaves>(p, 0, units(kSparseWaves), st);
+  if (p.nKt <= kShortMaxTiles && !p.long_key_kernel) return launch_variant<FP8, POW2, false, kShortWaves>(p, 0, units(kShortWaves), st);
   // Long dense call: one workgroup per CU at a time, so the call runs in rounds of `cus` workgroups.  When the
   // last round would be less than two thirds full, its query tiles go to the SPLIT form instead (three
   // workgroups of a third of the duration each per tile), launched behind the whole rounds.
@@ -810,10 +832,10 @@ static void launch_fp(const FwdParams& p, int cus, hipStream_t st) {
   const int whole = cus > 0 ? n / cus * cus : n, rest = n - whole;
   constexpr int kGroups = kDenseWaves / kShortWaves;
   if (whole > 0 && rest > 0 && rest * kGroups <= 2 * cus && !p.long_key_kernel) {
-    launch_variant<FP8, false, kDenseWaves>(p, 0, whole, st);
-    launch_variant<FP8, false, kDenseWaves, true>(p, whole * kGroups, rest * kGroups, st);
+    launch_variant<FP8, POW2, false, kDenseWaves>(p, 0, whole, st);
+    launch_variant<FP8, POW2, false, kDenseWaves, true>(p, whole * kGroups, rest * kGroups, st);
   } else {
-    launch_variant<FP8, false, kDenseWaves>(p, 0, n, st);
+    launch_variant<FP8, POW2, false, kDenseWaves>(p, 0, n, st);
   }
 }
 
@@ -840,7 +862,8 @@ hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
   int cus = 0;
   hipError_t e = device_cu_count(&cus);
   if (e != hipSuccess) return e;
-  if (p.fp8) launch_fp<true>(p, cus, st);
+  if (p.fp8 && p.fp8_pow2) launch_fp<true, true>(p, cus, st);
+  else if (p.fp8) launch_fp<true>(p, cus, st);
   else launch_fp<false>(p, cus, st);
   return hipGetLastError();
 }

@@ -163,6 +163,23 @@ __device__ __forceinline__ int k8_chunk_offset(int rt, int p8) {
 // key (inside its 32-key half) that element j of lane group g carries in a V image / in the P operand
 __device__ __forceinline__ int v_image_key(int g, int j) { return 16 * (j >> 2) + 4 * g + (j & 3); }
 
+// Dequantisation scale of an fp8 block whose largest magnitude is `amax`: amax / 448, or, with `pow2`, the smallest
+// power of two that is at least that (the form the scaled MFMA takes as an operand: an 8-bit exponent).  The product
+// amax * fl(1/448) is rounded to float32 first and the power of two is taken of that number.  A block of zeros gets 1.
+__device__ __forceinline__ float fp8_block_scale(float amax, bool pow2) {
+  if (!(amax > 0.f)) return 1.0f;
+  const float s = amax * (1.0f / kFp8Max);
+  if (!pow2) return s;
+  const unsigned bits = __float_as_uint(s);
+  unsigned e = (bits >> 23) & 0xffu;
+  if (bits & 0x7fffffu) ++e;
+  e = e < 1u ? 1u : (e > 254u ? 254u : e);
+  return __uint_as_float(e << 23);
+}
+
+// the 8-bit exponent (E8M0: value 2^(e - 127)) of a power-of-two scale, as the scaled MFMA takes it
+__device__ __forceinline__ int e8m0_of(float pow2_scale) { return (int)((__float_as_uint(pow2_scale) >> 23) & 0xffu); }
+
 // values 16*c .. 16*c+15 of a lane's row -> 16 bytes of fp8 e4m3: pieces ks8 = 2c (words 0, 1) and 2c + 1 (words 2, 3)
 __device__ __forceinline__ i32x4 quant_fp8_chunk(const float (&x)[64], int c, float inv) {
   i32x4 t;

@@ -374,7 +374,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
           }
       } else {
         amax = wave_max(amax);
-        const float scale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
+        const float scale = fp8_block_scale(amax, tg.fp8_pow2 != 0);
         const float inv = 1.0f / scale;
         if (lane == 0) tg.scale_out[(int64_t)head * tg.scale_head_stride + tile] = scale;
         // fp8 K tile: key block t is 2 KiB, chunk c2 of a lane holds its pieces ks = 2*c2 and 2*c2 + 1

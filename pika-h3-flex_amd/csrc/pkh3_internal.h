@@ -39,6 +39,7 @@ struct QkPrologueParams {
   int out_blk_stride;       // bytes between consecutive 64-row blocks
   float* scale_out;         // fp8: [B*H, nBlk64] dequantisation scales, else null
   int fp8;
+  int fp8_pow2;             // fp8: block scales rounded up to a power of two
   unsigned* norm_max;       // [B*H] float bits: max row norm after norm+rotation (atomic max), or null
 };
 
@@ -79,6 +80,7 @@ struct FwdParams {
   const float* kscale;      // [B*H, nKt] fp8 dequantisation scales of the K tiles
   const float* kmax;        // [B*H] largest K' row norm
   int fp8;
+  int fp8_pow2;         // fp8: the block scales are powers of two and ride in the scaled MFMA's operands
   int long_key_kernel;  // only the plain long-key form (no short-key form, no split last round)
   int unit0, units;     // filled per launch: the workgroup units [unit0, unit0 + units) this launch covers
 };
@@ -118,6 +120,7 @@ struct GemmTarget {
   const float* sin_t;
   unsigned* norm_max;      // [heads] float bits, atomic max of the row norms, or null
   int fp8;
+  int fp8_pow2;            // fp8: block scales rounded up to a power of two
   float* scale_out;        // fp8: [heads][scale_head_stride] dequantisation scales
   int scale_head_stride;
   // kEpiRows: y = residual + gate[row_index[token]] * (acc * out_scale + bias)

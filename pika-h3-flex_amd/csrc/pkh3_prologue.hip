@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
 #pragma unroll
       for (int i = 0; i < 64; ++i) amax = fmaxf(amax, fabsf(x[sub][i]));
     amax = wave_max(amax);
-    const float scale = amax > 0.f ? amax * (1.0f / kFp8Max) : 1.0f;
+    const float scale = fp8_block_scale(amax, p.fp8_pow2 != 0);
     const float inv = 1.0f / scale;
     if (lane == 0) p.scale_out[(int64_t)(b * p.H + h) * p.nBlk64 + blk] = scale;
 #pragma unroll

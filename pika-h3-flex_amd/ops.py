@@ -67,6 +67,20 @@ def _f32(name: str, t: Optional[torch.Tensor], shape, device) -> Optional[torch.
     return t
 
 
+FP8_POW2 = "pow2"  # value of ``fp8_qk`` that selects power-of-two block scales (PKH3_FLAG_FP8_POW2_SCALES)
+
+
+def fp8_mode(fp8_qk) -> object:
+    """Normal form of the ``fp8_qk`` option: False, True (absmax / 448 scales) or ``"pow2"`` (every block scale
+    the smallest power of two >= absmax / 448, softmax scale folded into Q before quantisation: faster, same e4m3
+    rounding error)."""
+    if isinstance(fp8_qk, str):
+        if fp8_qk != FP8_POW2:
+            raise ValueError(f'fp8_qk must be False, True or "{FP8_POW2}", got {fp8_qk!r}')
+        return FP8_POW2
+    return bool(fp8_qk)
+
+
 def fill_args(
     q, k, v, out, *, q_norm_weight=None, k_norm_weight=None, norm_eps=1e-6, rope_q=None, rope_k=None,
     rope_mode=_lib.ROPE_NONE, key_mask=None, block_mask: Optional[BlockMask] = None, fp8_qk=False,
@@ -76,6 +90,7 @@ def fill_args(
     """Build ``pkh3_attn_args`` for these tensors.  Returns (args, keep_alive).  ``kv_prepared``: K and V
     come through the workspace, from the fused projection (``pkh3_qkv_proj``) or from ``pkh3_kv_prepare``
     (then ``prepared_keys`` is their Sk); ``k`` and ``v`` are then None.
+    ``fp8_qk``: False, True or ``"pow2"`` (see :func:`fp8_mode`).
     ``out_images``: ``out`` is a uint8 operand-image buffer for ``pkh3_out_proj`` (``projections.packed_bytes(Sq,
     H*D)`` bytes) instead of a ``[B, Sq, H, D]`` tensor, and B must be 1."""
     if kv_prepared != (k is None) or (k is None) != (v is None):
@@ -145,7 +160,9 @@ def fill_args(
             raise ValueError("block mask CSR arrays must be contiguous")
         a.blk_row_ptr, a.blk_col_idx = block_mask.row_ptr.data_ptr(), block_mask.col_idx.data_ptr()
         keep += [block_mask.row_ptr, block_mask.col_idx]
-    a.flags = ((_lib.FLAG_FP8_QK if fp8_qk else 0) | (_lib.FLAG_LONG_KEY_KERNEL if long_key_kernel else 0)
+    fp8_qk = fp8_mode(fp8_qk)
+    a.flags = ((_lib.FLAG_FP8_QK if fp8_qk else 0) | (_lib.FLAG_FP8_POW2_SCALES if fp8_qk == FP8_POW2 else 0)
+               | (_lib.FLAG_LONG_KEY_KERNEL if long_key_kernel else 0)
                | (_lib.FLAG_KV_PREPARED if kv_prepared else 0) | (_lib.FLAG_O_IMAGES if out_images else 0))
     keep += [qw, kw]
     return a, keep

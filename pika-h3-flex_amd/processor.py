@@ -19,7 +19,7 @@ from typing import Dict, Hashable, Optional, Tuple
 import torch
 
 from . import _lib
-from .ops import BlockMask, PreparedKV, attention, attention_prepared, prepare_kv, rope_tables
+from .ops import BlockMask, PreparedKV, attention, attention_prepared, fp8_mode, prepare_kv, rope_tables
 from .projections import PackedLinear, adaln_modulate, out_proj, pack_rows, qkv_attention
 
 
@@ -84,7 +84,7 @@ class PikaH3AttnProcessor:
         rope_axes_dims: Tuple[int, int, int] = (32, 48, 48),
         rope_theta: float = 10000.0,
         norm_eps: float = 1e-6,
-        fp8_qk: bool = False,
+        fp8_qk=False,
         fused_projections: bool = False,
         lora_adapter: str = "default",
         cache_cross_kv: bool = False,
@@ -94,7 +94,7 @@ class PikaH3AttnProcessor:
         self.rope_axes_dims = tuple(int(x) for x in rope_axes_dims)
         self.rope_theta = float(rope_theta)
         self.norm_eps = float(norm_eps)
-        self.fp8_qk = bool(fp8_qk)
+        self.fp8_qk = fp8_mode(fp8_qk)  # False, True or "pow2"
         # self-attention of one document through the library's own projection GEMMs (LoRA as a second K segment,
         # K/V written by the GEMM epilogue in the attention kernel's layout) instead of the module's torch GEMMs
         self.fused_projections = bool(fused_projections)
@@ -183,7 +183,7 @@ class PikaH3AttnProcessor:
         cannot be reused).  Either way the key also holds the identity and version of the module's K-side weights
         (adapters included), so training steps or a swapped adapter prepare the keys again.  The cache is bounded by
         the bytes of its workspaces (``cross_kv_cache_bytes``), oldest entries dropped first."""
-        common = (float(k_opts["norm_eps"]), bool(k_opts["fp8_qk"]), tuple(enc.shape), str(enc.device), self._weights_state(attn))
+        common = (float(k_opts["norm_eps"]), str(k_opts["fp8_qk"]), tuple(enc.shape), str(enc.device), self._weights_state(attn))
         if cache_key is not None:
             key = (id(attn), "key", cache_key) + common
         else:
@@ -217,7 +217,7 @@ class PikaH3AttnProcessor:
         position_ids: Optional[torch.Tensor] = None,
         rope_cos_sin: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
         block_mask: Optional[BlockMask] = None,
-        fp8_qk: Optional[bool] = None,
+        fp8_qk=None,
         rope_key: Optional[Hashable] = None,
         adaln: Optional[dict] = None,
         gate: Optional[torch.Tensor] = None,
@@ -264,7 +264,7 @@ class PikaH3AttnProcessor:
         eps = getattr(qn, "eps", None)
         eps = self.norm_eps if eps is None else float(eps)
         scale = getattr(attn, "scale", None)
-        use_fp8 = (self.fp8_qk if fp8_qk is None else bool(fp8_qk)) and attention_mask is None
+        use_fp8 = (self.fp8_qk if fp8_qk is None else fp8_mode(fp8_qk)) if attention_mask is None else False
         q = attn.to_q(hidden_states)
         D = q.shape[-1] // H
         # [B, S, H*D] -> [B, S, H, D] views: no transpose copy, the kernels take the strides
@@ -328,7 +328,7 @@ class PikaH3AttnProcessor:
         opts = dict(
             q_norm_weight=_norm_weight(qn, 128, x.device), k_norm_weight=_norm_weight(kn, 128, x.device),
             norm_eps=self.norm_eps if eps is None else float(eps),
-            fp8_qk=self.fp8_qk if fp8_qk is None else bool(fp8_qk), block_mask=block_mask,
+            fp8_qk=self.fp8_qk if fp8_qk is None else fp8_mode(fp8_qk), block_mask=block_mask,
             softmax_scale=None if scale is None else float(scale),
         )
         if rope_cos_sin is None and position_ids is not None:

@@ -22,7 +22,7 @@ def test_header_symbols_are_exported(lib):
 
 
 def test_version_and_strerror(lib):
-    assert lib.pkh3_version() == 106
+    assert lib.pkh3_version() == 107
     assert lib.pkh3_strerror(0) == b"ok"
     assert b"128" in lib.pkh3_strerror(_lib.PKH3_EHEADDIM)
 
@@ -83,6 +83,7 @@ def test_workspace_bytes_host_only(lib):
     (lambda a: setattr(a, "workspace", 0x100010), _lib.PKH3_EWORKSPACE),
     (lambda a: setattr(a, "workspace_bytes", 1024), _lib.PKH3_EWORKSPACE),
     (lambda a: setattr(a, "flags", 0x80), _lib.PKH3_EARG),
+    (lambda a: setattr(a, "flags", _lib.FLAG_FP8_POW2_SCALES), _lib.PKH3_EARG),   # an option of FLAG_FP8_QK only
     (lambda a: setattr(a, "rope_mode", 7), _lib.PKH3_EARG),
     (lambda a: setattr(a, "rope_mode", 1), _lib.PKH3_ENULL),          # tables missing
     (lambda a: setattr(a, "blk_row_ptr", 0x20000), _lib.PKH3_ENULL),  # col_idx missing

@@ -38,7 +38,7 @@ def _oracle_rows(inp, rows, *, tabs=None, tile_map=None, fp8=False, heads=HEADS_
     if tile_map is not None:
         kw.update(tile_map=tile_map)
     if fp8:
-        kw.update(fp8_qk=True)
+        kw.update(fp8_qk=fp8)   # True or "pow2"
     return O.reference_layer(q, k, v, **kw)
 
 
@@ -87,7 +87,7 @@ def _oracle_full(inp, *, tile_map=None, fp8=False, heads=None, norm_w=None, bf16
     if tile_map is not None:
         kw.update(tile_map=tile_map)
     if fp8:
-        kw.update(fp8_qk=True)
+        kw.update(fp8_qk=fp8)   # True or "pow2"
     if bf16_operands:
         kw.update(bf16_operands=True)
     outs = []
@@ -218,6 +218,29 @@ def test_480p_full_tensor_block_sparse_and_fp8(inp480):
     _check_full(out8, _oracle_full(inp480, tile_map=tm, fp8=True), max_abs=1.0, min_cos=0.995, min_row_cos=0.98,
                 rel_abs=0.05, label="480p sparse fp8 vs fp8 oracle")
     for extra in (dict(block_mask=bm), dict(block_mask=bm, fp8_qk=True)):
+        mass = _indicator_mass(inp480, **extra)
+        assert float((mass - 1.0).abs().max()) < 1.5e-2, extra.keys()
+
+
+def test_480p_full_tensor_fp8_pow2_scales(inp480):
+    """The opt-in quantisation rule (power-of-two block scales applied by the matrix instruction, softmax scale
+    folded into Q before quantisation), dense and block-sparse, over every row and head against the oracle with the
+    same rule; its distance to the absmax-scale oracle and to the unquantised one is printed beside it."""
+    import pika_h3_flex_amd as pk
+
+    S = inp480.q.shape[1]
+    out8, _, _ = _run(inp480, fp8_qk="pow2")
+    _check_full(out8, _oracle_full(inp480, fp8="pow2"), max_abs=1.0, min_cos=0.995, min_row_cos=0.98, rel_abs=0.05,
+                label="480p fp8 pow2 vs pow2 oracle")
+    _check_full(out8, _oracle_full(inp480, fp8=True), max_abs=1.0, min_cos=0.995, min_row_cos=0.95, label="480p fp8 pow2 vs absmax oracle")
+    _check_full(out8, _oracle_full(inp480), max_abs=1.0, min_cos=0.995, min_row_cos=0.95, label="480p fp8 pow2 vs unquantised oracle")
+    del out8
+    tm = pk.local_window_tile_map(S, inp480.tokens_per_frame, window_frames=2, global_fraction=0.10, seed=0)
+    bm = pk.BlockMask.from_dense(tm, device="cuda")
+    outs, _, _ = _run(inp480, block_mask=bm, fp8_qk="pow2")
+    _check_full(outs, _oracle_full(inp480, tile_map=tm, fp8="pow2"), max_abs=1.0, min_cos=0.995, min_row_cos=0.98,
+                rel_abs=0.05, label="480p sparse fp8 pow2 vs pow2 oracle")
+    for extra in (dict(fp8_qk="pow2"), dict(block_mask=bm, fp8_qk="pow2")):
         mass = _indicator_mass(inp480, **extra)
         assert float((mass - 1.0).abs().max()) < 1.5e-2, extra.keys()
 

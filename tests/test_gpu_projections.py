@@ -117,7 +117,7 @@ def _packed(d, head_perm=True):
 
 @pytest.mark.parametrize("S,H,variant", [
     (300, 2, "bf16"), (777, 3, "bf16"), (64, 1, "bf16"), (1000, 2, "no_lora"), (520, 2, "fp8"), (700, 2, "sparse"),
-    (450, 3, "rope_half"),
+    (450, 3, "rope_half"), (520, 2, "fp8_pow2"),
 ])
 def test_qkv_projection_feeds_attention(S, H, variant):
     """to_q/to_k/to_v (+LoRA, bias) with the K-side norm + rotation and the K/V layout in the GEMM epilogue, then the
@@ -139,6 +139,9 @@ def test_qkv_projection_feeds_attention(S, H, variant):
     if variant == "fp8":
         opts.update(fp8_qk=True)
         ref_opts.update(fp8_qk=True)
+    if variant == "fp8_pow2":   # the K epilogue of the GEMM forms the power-of-two scales
+        opts.update(fp8_qk="pow2")
+        ref_opts.update(fp8_qk="pow2")
     if variant == "sparse":
         n = (S + 63) // 64
         tm = (torch.rand((n, n), generator=torch.Generator().manual_seed(3)) < 0.5) | torch.eye(n, dtype=torch.bool)
@@ -159,7 +162,7 @@ def test_qkv_projection_feeds_attention(S, H, variant):
     err, cos = AO.max_abs_and_cosine(out.cpu(), o_ref)
     print(f"[{variant} S={S} H={H}] O: max_abs={err:.3e} cos={cos:.8f}", flush=True)
     assert torch.isfinite(out.float()).all()
-    if variant == "fp8":
+    if variant.startswith("fp8"):
         assert cos >= 0.995
     else:
         assert err <= 2e-2 and cos >= 0.9999
@@ -167,7 +170,7 @@ def test_qkv_projection_feeds_attention(S, H, variant):
     unfused = pk.attention(r(q_ref).cuda(), r(k_ref).cuda(), r(v_ref).cuda(), **opts)
     torch.cuda.synchronize()
     err, cos = AO.max_abs_and_cosine(out.cpu(), unfused.cpu())
-    assert cos >= (0.995 if variant == "fp8" else 0.9999)
+    assert cos >= (0.995 if variant.startswith("fp8") else 0.9999)
 
 
 @pytest.mark.parametrize("S,N,K,lora,extras", [(300, 256, 256, True, True), (1000, 384, 256, False, True), (65, 128, 512, True, False)])

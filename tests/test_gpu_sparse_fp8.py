@@ -159,3 +159,82 @@ def test_sparse_and_fp8_with_large_logits():
     err8, cos8 = O.max_abs_and_cosine(out8, ref8)
     print(f"fp8 large logits: max_abs={err8:.3e} cos={cos8:.6f}", flush=True)
     assert cos8 >= 0.995
+
+
+@pytest.mark.parametrize("long_form", [False, True])
+@pytest.mark.parametrize("Sq,Sk,rope,scale", [(256, 256, 0, None), (1000, 1000, 1, None), (777, 1500, 2, 0.2), (300, 5000, 1, 0.05)])
+def test_fp8_pow2_scales(Sq, Sk, rope, scale, long_form):
+    """fp8_qk="pow2" (power-of-two block scales inside the scaled MFMA, softmax scale folded into Q before the
+    quantisation) against the oracle with the same rule: the short-key and the long-key forms, rectangular calls
+    with their own key tables, other softmax scales."""
+    from oracle import attention_oracle as O
+
+    q, k, v, gen = _inputs(2, Sq, Sk, 2, seed=300 + Sq)
+    w = torch.ones(D)
+    opts, ref_opts = {}, {}
+    if rope:
+        tq = O.rope_tables(torch.rand((Sq, 3), generator=gen, dtype=torch.float64) * 30.0)
+        tk = tq if Sq == Sk else O.rope_tables(torch.rand((Sk, 3), generator=gen, dtype=torch.float64) * 30.0)
+        ref_opts = dict(rope_q=tq, rope_k=tk, rope_mode=rope)
+        dev = lambda t: tuple(x.float().contiguous().cuda() for x in t)
+        opts = dict(rope_q=dev(tq), rope_k=dev(tk), rope_mode=rope)
+    ref8 = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, fp8_qk="pow2", scale=scale, **ref_opts)
+    ref = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, scale=scale, **ref_opts)
+    out = _call(q, k, v, q_norm_weight=_ones(), k_norm_weight=_ones(), fp8_qk="pow2", long_key_kernel=long_form,
+                softmax_scale=scale, **opts)
+    err8, cos8 = O.max_abs_and_cosine(out, ref8)
+    err, cos = O.max_abs_and_cosine(out, ref)
+    print(f"fp8 pow2 Sq={Sq} Sk={Sk} rope={rope} scale={scale}: vs pow2 oracle max_abs={err8:.3e} cos={cos8:.6f}; "
+          f"vs unquantised max_abs={err:.3e} cos={cos:.6f}", flush=True)
+    assert cos8 >= 0.995
+    # the emulation is followed much more tightly than the contract asks (sharper softmax scales give larger outputs)
+    assert cos8 >= 0.9995 and err8 <= 2e-2 * max(1.0, float(ref8.abs().max()))
+    assert cos >= 0.995
+
+
+def test_fp8_pow2_block_sparse_large_logits_and_zero_rows():
+    """The same rule through the block-sparse kernel, through the running-max softmax (norm weight 4), and on
+    all-zero Q and K blocks (scale 1, exponent byte 127: finite outputs, zero logits)."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as O
+
+    q, k, v, gen = _inputs(1, 900, 900, 2, seed=41)
+    tm = _tile_map(15, 15, 0.3, gen)
+    w = torch.ones(D)
+    ref8 = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, fp8_qk="pow2", tile_map=tm)
+    out = _call(q, k, v, q_norm_weight=_ones(), k_norm_weight=_ones(), fp8_qk="pow2",
+                block_mask=pk.BlockMask.from_dense(tm, device="cuda"))
+    err8, cos8 = O.max_abs_and_cosine(out, ref8)
+    print(f"fp8 pow2 + sparse: max_abs={err8:.3e} cos={cos8:.6f}", flush=True)
+    assert cos8 >= 0.9995 and err8 <= 2e-2
+
+    w4 = torch.full((D,), 4.0)
+    for extra, rex in ((dict(), dict()), (dict(block_mask=pk.BlockMask.from_dense(tm, device="cuda")), dict(tile_map=tm))):
+        ref = O.reference_layer(q, k, v, q_norm_weight=w4, k_norm_weight=w, fp8_qk="pow2", **rex)
+        out = _call(q, k, v, q_norm_weight=w4.cuda(), k_norm_weight=_ones(), fp8_qk="pow2", **extra)
+        err, cos = O.max_abs_and_cosine(out, ref)
+        print(f"fp8 pow2 large logits {list(extra)}: max_abs={err:.3e} cos={cos:.6f}", flush=True)
+        assert cos >= 0.995
+
+    qz, kz = q.clone(), k.clone()
+    qz[:, 64:128] = 0
+    kz[:, 128:192] = 0
+    ref = O.reference_layer(qz, kz, v, fp8_qk="pow2")
+    out = _call(qz, kz, v, fp8_qk="pow2")
+    assert torch.isfinite(out.float()).all()
+    err, cos = O.max_abs_and_cosine(out, ref)
+    assert cos >= 0.9995 and err <= 2e-2
+    # an all-zero query block attends uniformly: its rows are the mean of V
+    mean_v = v.double().mean(dim=1, keepdim=True)
+    assert float((out[:, 64:128].double() - mean_v).abs().max()) <= 2e-2
+
+
+def test_fp8_pow2_prepared_keys_agree_with_the_direct_call():
+    import pika_h3_flex_amd as pk
+
+    q, k, v, gen = _inputs(1, 500, 1300, 2, seed=51)
+    direct = _call(q, k, v, q_norm_weight=_ones(), k_norm_weight=_ones(), fp8_qk="pow2")
+    kv = pk.prepare_kv(k.cuda(), v.cuda(), k_norm_weight=_ones(), fp8_qk="pow2")
+    out = pk.attention_prepared(q.cuda(), kv, q_norm_weight=_ones())
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), direct)

@@ -134,3 +134,12 @@ def test_key_padding_mask_forms():
     with pytest.raises(ValueError, match="additive"):
         key_padding_mask(torch.full((2, 5), float("nan")), 2, 5)
     assert torch.equal(key_padding_mask(torch.where(keep, 0.0, -1e3), 2, 5), keep)
+
+
+def test_fp8_option_forms():
+    from pika_h3_flex_amd.ops import fp8_mode
+
+    assert fp8_mode(False) is False and fp8_mode(None) is False and fp8_mode(True) is True and fp8_mode(1) is True
+    assert fp8_mode("pow2") == "pow2"
+    with pytest.raises(ValueError):
+        fp8_mode("e5m2")

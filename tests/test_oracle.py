@@ -247,6 +247,68 @@ def test_fake_quant_blocks_scales_and_error_bound():
     assert abs(float(deq[0, :64, 0].flatten()[i]) - float(x[0, :64, 0].flatten()[i])) < 1e-5 * float(x[0, :64, 0].abs().max())
 
 
+def test_pow2_ceil_over_every_float32_exponent():
+    """The bit rule against math.frexp (an independent path: frexp returns m in [0.5, 1) and e with x = m * 2^e, so
+    the smallest power of two >= x is 2^(e-1) when m == 0.5 and 2^e otherwise), on every normal exponent: the power
+    itself, one ulp above, one ulp below, and a mid-binade value."""
+    vals = []
+    for e in range(-126, 128):
+        p = np.float32(2.0) ** np.float32(e)
+        vals += [p, np.nextafter(p, np.float32(np.inf)), np.float32(p * np.float32(1.5))]
+        if e > -126:
+            vals.append(np.nextafter(p, np.float32(0)))
+    vals = np.array([v for v in vals if np.isfinite(v)], dtype=np.float32)
+    got = O.pow2_ceil_f32(torch.from_numpy(vals)).numpy().astype(np.float64)
+    for v, g in zip(vals.astype(np.float64), got):
+        m, e = math.frexp(float(v))
+        want = math.ldexp(1.0, e - 1 if m == 0.5 else e)
+        want = min(want, 2.0 ** 127)     # the largest scale an 8-bit exponent names
+        assert g == want, (v, g, want)
+        assert g >= min(v, 2.0 ** 127) and (g / 2 < v or g == 2.0 ** -126)
+
+
+def test_fake_quant_pow2_scales():
+    x = _r(1, 130, 2, 128, seed=29) * 3.0
+    x[0, 64:128, 1] = 0.0                      # a block of zeros: scale 1, values 0
+    x[0, 0, 0, 0] = 448.0 * 2.0 ** -5          # absmax / 448 an exact power of two: the scale is that power
+    x[0, :64, 0] = x[0, :64, 0].clamp(-14.0, 14.0)
+    deq, scales = O.fake_quant_fp8_blocks(x, pow2_scales=True)
+    ref_deq, ref_scales = O.fake_quant_fp8_blocks(x)
+    assert float(scales[0, 0, 0]) == 2.0 ** -5 and float(scales[0, 1, 1]) == 1.0
+    assert torch.count_nonzero(deq[0, 64:128, 1]) == 0
+    for blk, h in itertools.product(range(3), range(2)):
+        s = float(scales[0, h, blk])
+        rows = x[0, blk * 64 : (blk + 1) * 64, h].double()
+        if float(rows.abs().max()) == 0:
+            continue
+        m, e = math.frexp(s)
+        assert m == 0.5                                             # a power of two
+        assert float(ref_scales[0, h, blk]) <= s < 2 * float(ref_scales[0, h, blk])
+        # brute force: the nearest e4m3 value of rows / s, scaled back (division by a power of two is exact)
+        want = torch.from_numpy(O.fp8_e4m3_round((rows / s).numpy())) * s
+        assert torch.equal(deq[0, blk * 64 : (blk + 1) * 64, h], want)
+        assert float((rows / s).abs().max()) <= 448.0               # nothing saturates
+        err = (want - rows).abs()
+        assert bool((err <= torch.maximum(rows.abs() * 2.0 ** -4, torch.tensor(s * 2.0 ** -10)) * (1 + 1e-9)).all())
+
+
+def test_reference_layer_pow2_folds_the_softmax_scale_into_q():
+    """fp8_qk="pow2": K as fake_quant(pow2), Q as fake_quant(pow2) of q * scale * log2(e), divided back."""
+    q, k, v = _r(1, 96, 2, 128, seed=30), _r(1, 80, 2, 128, seed=31), _r(1, 80, 2, 128, seed=32)
+    w = torch.ones(128)
+    got = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, fp8_qk="pow2", scale=0.11)
+    cq = float(np.float32(0.11) * np.float32(1.4426950408889634))
+    qn, kn = O.rms_norm(q, w, 1e-6), O.rms_norm(k, w, 1e-6)
+    qd = O.fake_quant_fp8_blocks(qn.float() * cq, pow2_scales=True)[0] / cq
+    kd = O.fake_quant_fp8_blocks(kn, pow2_scales=True)[0]
+    want = O.attention(qd, kd, v, scale=0.11)
+    assert torch.equal(got, want)
+    # and it stays an fp8-grade approximation of the unquantised layer, like the absmax form
+    plain = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, scale=0.11)
+    absmax = O.reference_layer(q, k, v, q_norm_weight=w, k_norm_weight=w, fp8_qk=True, scale=0.11)
+    assert O.max_abs_and_cosine(got, plain)[1] >= 0.999 and O.max_abs_and_cosine(absmax, plain)[1] >= 0.999
+
+
 def test_reference_layer_composes_the_parts():
     S = 40
     q, k, v = (_r(1, S, 2, 128, seed=s).to(torch.bfloat16) for s in (30, 31, 32))
