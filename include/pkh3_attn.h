@@ -86,9 +86,11 @@ enum {
                                  the e4m3 range is given up; the error stays that of an e4m3 rounding (relative step
                                  2^-4) */
   PKH3_FLAG_LONG_KEY_KERNEL = 1u << 1 /* dense calls with at most 16 key tiles (Sk <= 1024) normally run a
-                                 short-key form of the kernel (small workgroups, three per CU); this flag
-                                 selects the long-key form for them too.  Same results to the tolerance of the
-                                 path; meant for tests and measurements */
+                                 short-key form of the kernel (small workgroups, three per CU), and long dense
+                                 calls share the query tiles of a thinly filled last round of workgroups out
+                                 among several workgroups each; this flag selects the plain long-key form,
+                                 one workgroup per query tile, for all of them.  Same results to the tolerance
+                                 of the path; meant for tests and measurements */
 };
 
 typedef struct pkh3_attn_args {

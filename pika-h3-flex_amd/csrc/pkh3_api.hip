@@ -97,7 +97,7 @@ int validate(const pkh3_attn_args* a, bool pointers, bool caller_workspace = tru
   return PKH3_OK;
 }
 
-WsPlan plan(const pkh3_attn_args* a) {
+WsPlan plan(const pkh3_attn_args* a, bool part_scratch = true) {
   WsPlan w{};
   const bool fp8 = a->flags & PKH3_FLAG_FP8_QK;
   w.nQ64 = (int)align_up((size_t)(a->Sq + 63) / 64, 4);
@@ -114,6 +114,15 @@ WsPlan plan(const pkh3_attn_args* a) {
   // what follows depends on the queries of the call
   w.plan_off = off;   if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / kSparseRows) * kSparseLists * w.nKt * sizeof(int), 256);
   w.plan_cnt_off = off; if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / kSparseRows) * kSparseLists * sizeof(int), 256);
+  // long dense calls: partial results and arrival counters of the workgroups that may share out the units of the
+  // call's last round (none for short-key calls and for calls too small to fill a round of workgroups on any device;
+  // `part_scratch` false: none at all, the call then ends on whole workgroups)
+  const size_t tiles384 = bh * (((size_t)w.nQ64 * 2 + 11) / 12);
+  const size_t part_wgs = (!part_scratch || a->blk_row_ptr || w.nKt <= kShortMaxTiles || tiles384 < 64) ? 0
+                          : (tiles384 * 8 < (size_t)kMaxPartWorkgroups ? tiles384 * 8 : (size_t)kMaxPartWorkgroups);
+  w.split_bytes = part_wgs * 12 * (size_t)kPartialBytes;
+  w.split_off = off;  off = align_up(off + w.split_bytes, 256);
+  w.split_cnt_off = off; off = align_up(off + part_wgs * 12 * sizeof(int), 256);
   w.total = off;
   return w;
 }
@@ -128,9 +137,9 @@ struct Launch {
   int* idx;
 };
 
-void build(const pkh3_attn_args* a, void* workspace, Launch& L) {
+void build(const pkh3_attn_args* a, void* workspace, Launch& L, bool part_scratch = true) {
   const bool fp8 = a->flags & PKH3_FLAG_FP8_QK;
-  L.w = plan(a);
+  L.w = plan(a, part_scratch);
   L.ws = (char*)workspace;
   char* ws = L.ws;
   L.cnt = a->key_mask ? (int*)(ws + L.w.cnt_off) : nullptr;
@@ -176,6 +185,9 @@ void build(const pkh3_attn_args* a, void* workspace, Launch& L) {
   f.plan_stride = kSparseLists * L.w.nKt;
   f.kscale = k.scale_out; f.fp8 = fp8; f.fp8_pow2 = k.fp8_pow2; f.long_key_kernel = (a->flags & PKH3_FLAG_LONG_KEY_KERNEL) ? 1 : 0;
   f.kmax = (const float*)(ws + L.w.kmax_off);
+  f.split_scratch = L.w.split_bytes ? (float*)(ws + L.w.split_off) : nullptr;
+  f.split_scratch_bytes = L.w.split_bytes;
+  f.split_cnt = L.w.split_bytes ? (int*)(ws + L.w.split_cnt_off) : nullptr;
 }
 
 int hip_fail(hipError_t e, const char* what) {
@@ -342,7 +354,9 @@ int pkh3_attn_fwd_noalloc(const pkh3_attn_args* a, void* stream) {
   if (rc) return rc;
   if (a->flags & PKH3_FLAG_KV_PREPARED)
     return fail(PKH3_EUNSUPPORTED, "pkh3_attn_fwd_noalloc: prepared K/V live in a caller workspace, which this call does not take");
-  const size_t need = plan(a).total;
+  // the scratch of the shared last round (a matter of speed only) is left out when the built-in buffer cannot hold it
+  const bool part_scratch = plan(a, true).total <= (size_t)PKH3_NOALLOC_SCRATCH_BYTES;
+  const size_t need = plan(a, part_scratch).total;
   if (need > (size_t)PKH3_NOALLOC_SCRATCH_BYTES)
     return fail(PKH3_EWORKSPACE,
                 "pkh3_attn_fwd_noalloc: this call needs %zu bytes of scratch, the built-in buffer holds %zu; use "
@@ -351,7 +365,7 @@ int pkh3_attn_fwd_noalloc(const pkh3_attn_args* a, void* stream) {
   void* ptr = nullptr;  // this device's copy of the built-in scratch array
   if ((rc = static_scratch(&ptr))) return rc;
   Launch L;
-  build(a, ptr, L);
+  build(a, ptr, L, part_scratch);
   hipStream_t st = (hipStream_t)stream;
   if ((rc = run_prologue(a, L, st))) return rc;
   hipError_t e = launch_attn_fwd(L.f, st);

@@ -25,8 +25,8 @@
 // around into whole 256-byte rows.
 //
 // Other forms of the dense kernel (see attn_fwd_kernel): the short-key form (at most 16 key tiles: 4 waves per
-// workgroup, 32-key half tiles, three workgroups per CU) and the split form for a thinly filled last round of
-// a long call (128 queries per workgroup, its three groups of 4 waves walk a third of the keys each).
+// workgroup, 32-key half tiles, three workgroups per CU), and the long form with the key tiles of a unit shared out
+// among several workgroups that merge through global scratch, for a thinly filled last round of a long call.
 //
 // Block-sparse variant.  A workgroup covers 4 query row-blocks (64 queries each, a wave pair per row-block).
 // Phase 1 walks the key tiles all four row-blocks keep, exactly like the dense kernel.  Phase 2 walks the
@@ -41,7 +41,8 @@ namespace pkh3 {
 
 constexpr int kDenseWaves = 12;  // dense kernel: three waves per SIMD (<= 168 VGPRs each), 384 queries per workgroup
 constexpr int kShortWaves = 4;   // short-key dense kernel: three 4-wave workgroups per CU
-constexpr int kShortMaxTiles = 16;  // key tiles up to which the short-key kernel is used
+constexpr int kMaxParts = 8;     // long dense form: most workgroups a unit's key tiles are shared out among ...
+constexpr int kMinPartTiles = 24;  // ... and fewest key tiles such a workgroup is worth starting for
 constexpr int kSparseWaves = 2 * kSparseRows;  // block-sparse: a wave pair per row-block; two such workgroups share a CU
 constexpr int kRing = 3;               // LDS ring depth (tiles)
 constexpr float kRescaleSlack = 8.0f;  // the running max is only raised when exceeded by 2^8
@@ -81,6 +82,28 @@ __device__ __forceinline__ void lds_dma16(const char* g, unsigned lane_off, char
 template <typename T>
 __device__ __forceinline__ T uniform_load(const T* p, int i) {
   return ((const __attribute__((address_space(4))) T*)p)[i];
+}
+
+// Stores and loads that are coherent across the whole device (all XCDs) one by one: they go past the caches that
+// are not, so data handed from one workgroup to another needs no cache write-back or invalidation around it --
+// only the writer's wait for its stores before it signals, and the reader's signal check before its loads.
+__device__ __forceinline__ void store_device(float* p, f32x4 v) {
+  const unsigned long long lo = ((unsigned long long)__float_as_uint(v[1]) << 32) | __float_as_uint(v[0]);
+  const unsigned long long hi = ((unsigned long long)__float_as_uint(v[3]) << 32) | __float_as_uint(v[2]);
+  __hip_atomic_store((unsigned long long*)p, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store((unsigned long long*)p + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_device(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f32x4 load_device4(const float* p) {
+  const unsigned long long lo = __hip_atomic_load((const unsigned long long*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long hi = __hip_atomic_load((const unsigned long long*)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return f32x4{__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)), __uint_as_float((unsigned)hi),
+               __uint_as_float((unsigned)(hi >> 32))};
+}
+__device__ __forceinline__ float load_device(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // maximum over the four lanes l % 16 == const (one per 16-lane group): two row swaps, no LDS crossbar
@@ -362,14 +385,38 @@ __device__ __forceinline__ void softmax_pv_half(WaveState<FP8>& w, float c, int 
 // ring of 32-key half tiles in 48 KiB of LDS, so three workgroups share a CU and the Q load and O store of one
 // run under the tiles of the others.  With few key tiles that overlap is worth more than the three-fold K/V
 // copies cost (the K/V of such calls sit in L2).
-// SPLIT (dense, 12 waves) is the form for the last, partly filled round of a long dense call: the workgroup takes
-// 128 queries instead of 384 and its three groups of 4 waves walk one third of the keys each (half tiles, a ring
-// per group), then add their partial results up through LDS.  Such a workgroup lasts a third as long, so the
-// CUs that would idle through a whole round of whole workgroups idle through a third of one.
+// PARTS (long dense form only): `parts` workgroups share a unit's queries and walk 1/parts of the key tiles each, so
+// such a workgroup lasts 1/parts as long as a whole one: the way a call's last, thinly filled round of workgroups is
+// cut into pieces that fill the chip (see launch_fp).  Each wave leaves its partial result (un-normalised O^T, row
+// sums, row maxima) in global scratch; the wave that arrives last of the `parts` adds the others' to its own and
+// writes the output.
+constexpr int kMergeBytes = kPartialBytes;  // one wave's partial result in fp32
+
+// bytes of LDS a form of the kernel needs
+template <bool FP8, bool SPARSE, int WAVES>
+constexpr int fwd_lds_bytes() {
+  constexpr bool HALFMODE = !SPARSE && WAVES == kShortWaves;
+  constexpr int kRingT = (SPARSE && !FP8 && WAVES < 8) ? 2 : kRing;
+  constexpr int kStages2 = (SPARSE && FP8 && WAVES < 8) ? 3 : 2;
+  constexpr int kTileBytes = (FP8 ? kK8TileBytes : kKTileBytes) + kVTileBytes;
+  constexpr int kHalfBytes = kTileBytes / 2;
+  constexpr int kStageBytes = 32 * kD * 2;    // one wave's 32 x 128 bf16 output block, staged for the row-wise store
+  // dense / phase 1: ring of kRingT whole tiles; sparse phase 2: kStages2 stages of row-private half tiles
+  constexpr int kPhase2Bytes = SPARSE ? kStages2 * kSparseRows * kHalfBytes : 0;
+  constexpr int kRingBytes = HALFMODE ? kRing * kHalfBytes
+                             : (kPhase2Bytes > kRingT * kTileBytes ? kPhase2Bytes : kRingT * kTileBytes);
+  constexpr int kAfterBytes = WAVES * kStageBytes;  // LDS use after the loops
+  return kRingBytes > kAfterBytes ? kRingBytes : kAfterBytes;
+}
+
 // POW2 (fp8 only): power-of-two block scales, applied by the scaled MFMA; softmax_scale * log2(e) rides in Q' before
 // it is quantised, so the softmax has no multiply left (the instruction count of the bf16 form).
-template <bool FP8, bool SPARSE, int WAVES, bool SPLIT = false, bool POW2 = false>
-__global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWaves ? 3 : 1)) void attn_fwd_kernel(FwdParams p) {
+// One workgroup's work.  `blk`: index of the workgroup inside its section of the launch; the section covers the
+// units [unit0, unit0 + units), a unit being one workgroup's block of queries (`parts` workgroups per unit; their
+// partial results start at slot `part_base` of the scratch, their counters at unit slot `cnt_base`).
+template <bool FP8, bool SPARSE, int WAVES, bool POW2>
+__device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int unit0, int units, int parts, int part_base,
+                                              int cnt_base, char* lds_raw) {
   static_assert(!SPARSE || WAVES == kSparseWaves, "block-sparse layout: a wave pair per row-block of the plan");
   static_assert(FP8 || !POW2, "power-of-two scales belong to the fp8 form");
   constexpr bool SHORT = !SPARSE && WAVES == kShortWaves;
@@ -378,23 +425,13 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   constexpr int kRingT = (SPARSE && !FP8 && WAVES < 8) ? 2 : kRing;
   constexpr int kAhead = kRingT - 1;                    // tiles in flight ahead of the one being used
   constexpr int kStages2 = (SPARSE && FP8 && WAVES < 8) ? 3 : 2;  // sparse phase 2: stages of row-private half tiles
-  constexpr bool HALFMODE = SHORT || SPLIT;             // rings of 32-key half tiles, 4 waves per ring
-  constexpr int GROUPS = SPLIT ? WAVES / kShortWaves : 1;  // key-range groups of the workgroup
-  static_assert(!(HALFMODE && SPARSE), "the half-tile forms are dense only");
-  static_assert(!SPLIT || WAVES % kShortWaves == 0, "whole groups of 4 waves");
+  constexpr bool HALFMODE = SHORT;                      // ring of 32-key half tiles
+  constexpr bool PARTS = !SPARSE && !SHORT;             // the long dense form: the key tiles may be shared out (`parts`)
   constexpr int kKBytes = FP8 ? kK8TileBytes : kKTileBytes;
   constexpr int kTileBytes = kKBytes + kVTileBytes;
   constexpr int kChunks = kTileBytes / 1024;  // 1 KiB pieces of a tile, dealt round-robin to the waves
   constexpr int kHalfBytes = kTileBytes / 2;  // K and V images of 32 keys
-  // dense / phase 1: ring of kRingT whole tiles; sparse phase 2: kStages2 stages of row-private half tiles
   constexpr int kStageBytes = 32 * kD * 2;    // one wave's 32 x 128 bf16 output block, staged for the row-wise store
-  constexpr int kPhase2Bytes = SPARSE ? kStages2 * kSparseRows * kHalfBytes : 0;
-  constexpr int kRingBytes = HALFMODE ? GROUPS * kRing * kHalfBytes
-                             : (kPhase2Bytes > kRingT * kTileBytes ? kPhase2Bytes : kRingT * kTileBytes);
-  constexpr int kMergeBytes = 64 * 64 * 4 + 4 * 64 * 4;  // SPLIT: one wave's O^T, row sums and row maxima in fp32
-  constexpr int kAfterBytes = SPLIT ? kShortWaves * kMergeBytes : WAVES * kStageBytes;  // LDS use after the loops
-  constexpr int kLdsBytes = kRingBytes > kAfterBytes ? kRingBytes : kAfterBytes;
-  __shared__ __attribute__((aligned(1024))) char lds_raw[kLdsBytes];
   char(*lds)[kTileBytes] = (char(*)[kTileBytes])lds_raw;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -402,26 +439,19 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
 
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD one contiguous run of
   // (batch, head, query tile) so the 32 CUs behind one L2 stream the same K/V at the same time.
-  // A launch covers the units [p.unit0, p.unit0 + p.units); a unit is one workgroup's block of queries.
-  const int total = p.units;
+  // (Every section of a launch starts at a workgroup index that is a multiple of 8.)
+  const int total = units * parts;
   const int per_xcd = (total + 7) / 8;
-  const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int lin = (blk & 7) * per_xcd + (blk >> 3);
   if (lin >= total) return;
-  const int unit = p.unit0 + lin;
-  const int group = SPLIT ? wave / kShortWaves : 0;       // which third of the keys (SPLIT)
-  const int wq = HALFMODE ? wave % kShortWaves : wave;    // which 32-query block of the unit
-  int bh, qt, q32;
-  if constexpr (SPLIT) {
-    // units are thirds of the 12-wave form's query tiles, so that a call can hand its last tiles to this form
-    const int nQt = (p.nQ64 * 2 + WAVES - 1) / WAVES;
-    bh = (unit / GROUPS) / nQt, qt = (unit / GROUPS) % nQt;
-    q32 = qt * WAVES + (unit % GROUPS) * kShortWaves + wq;
-  } else {
-    constexpr int kBlocks = HALFMODE ? kShortWaves : WAVES;  // 32-query blocks per unit
-    const int nQt = (p.nQ64 * 2 + kBlocks - 1) / kBlocks;
-    bh = unit / nQt, qt = unit % nQt;
-    q32 = qt * kBlocks + wq;
-  }
+  // unit inside the section, and which share of its keys: share-major, so that the workgroups an XCD runs at the
+  // same time walk the same key tiles of (mostly) the same head, as the whole units before them do
+  const int part = lin / units, ul = lin % units;
+  const int unit = unit0 + ul;
+  const int wq = wave;                                    // which 32-query block of the unit
+  const int nQt = (p.nQ64 * 2 + WAVES - 1) / WAVES;       // units per (batch, head)
+  const int bh = unit / nQt, qt = unit % nQt;
+  const int q32 = qt * WAVES + wq;
   const int b = bh / p.H, h = bh % p.H;
 
   const int sk = p.row_cnt ? p.row_cnt[b] : p.Sk;
@@ -429,7 +459,11 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   // sparse: [tiles every row-block of this workgroup keeps | tiles only row-block 0 keeps | ... 1 | ...]
   const int* plan = SPARSE ? p.plan + (int64_t)qt * p.plan_stride : nullptr;
   const int* plan_cnt = SPARSE ? p.plan_cnt + qt * kSparseLists : nullptr;
-  const int nt = SPARSE ? uniform_load(plan_cnt, 0) : nkt;  // tiles all 8 waves walk together
+  const int nt = SPARSE ? uniform_load(plan_cnt, 0) : nkt;  // tiles all the waves walk together
+  // the tiles [t_begin, t_end) of those are this workgroup's share
+  // (32-bit arithmetic: at most 2^18 tiles times kMaxParts; the results address the tile copies from scalar registers)
+  const int t_begin = PARTS ? __builtin_amdgcn_readfirstlane(part * nt / parts) : 0;
+  const int t_end = PARTS ? __builtin_amdgcn_readfirstlane((part + 1) * nt / parts) : nt;
 
   // this wave's pieces of every [K|V] tile record: 1 KiB chunks wave, wave + WAVES, ...
   const char* kv_w = p.kv + (int64_t)bh * p.kv_bh_stride + wave * 1024;
@@ -443,13 +477,11 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   };
   auto entry = [&](int i) { return SPARSE ? uniform_load(plan, i) : i; };  // i-th shared tile
 
-  // half-tile forms: [K half | V half] per ring slot, one ring per group of 4 waves, every wave of the group
-  // copies the same share; group g walks the halves [h_begin, h_begin + n_mine)
+  // half-tile form: [K half | V half] per ring slot, every wave copies the same share
   constexpr int kKHalfB = kKBytes / 2, kVHalfB = kVTileBytes / 2;
   const int n_half = (sk + 31) / 32;
-  const int h_begin = group * n_half / GROUPS;
-  const int n_mine = (group + 1) * n_half / GROUPS - h_begin;
-  char* ring = lds_raw + group * (kRing * kHalfBytes);
+  const int h_begin = 0, n_mine = n_half;
+  char* ring = lds_raw;
   auto dma_short = [&](int half, int slot) {
     static_assert((kKHalfB / 1024) % kShortWaves == 0 && (kVHalfB / 1024) % kShortWaves == 0, "equal shares");
     const char* g = p.kv + (int64_t)bh * p.kv_bh_stride + (int64_t)(half >> 1) * p.kv_tile_stride;
@@ -471,9 +503,9 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   if constexpr (HALFMODE) {
     if (n_mine > 0) dma_short(h_begin, 0);
     if (n_mine > 1) dma_short(h_begin + 1, 1);
-  } else if (nt > 0) {
-    dma(entry(0), 0);
-    if (kAhead > 1 && nt > 1) dma(entry(1), 1);
+  } else if (t_end > t_begin) {
+    dma(entry(t_begin), 0);
+    if (kAhead > 1 && t_end > t_begin + 1) dma(entry(t_begin + 1), 1);
   }
   // Q load, fused with QK-RMSNorm, rotation and (fp8) quantisation: lane (l%32, hh) reads the 64 elements
   // d = 16*ks + 8*hh + j of query row q32*32 + l%32 (whole 8-element pieces of the MFMA B images), so the
@@ -586,7 +618,7 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   // Only the last key tile can be partial.  It is peeled off the loop so that the loop body has no masking
   // branch between S^T and the softmax, which lets the numerators of the first 32 keys be scheduled under
   // the MFMAs of the second 32.
-  const int n_masked = (tail && nt > 0 && entry(nt - 1) == nkt - 1) ? 1 : 0;
+  const int n_masked = (tail && t_end > t_begin && entry(t_end - 1) == nkt - 1) ? 1 : 0;
 #define PKH3_TILE_LOOP(STATIC, MASKED, FROM, TO)                                                        \
   for (int i = FROM; i < TO; ++i) {                                                                     \
     /* tile i (and, with a ring of three, i+1) is in LDS for every wave (own slices: vmcnt, the others': */ \
@@ -599,15 +631,14 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     qk_tile<FP8, LEAN, (MASKED) ? 2 : 4, POW2>(w, kbuf, kbuf + kKBytes, lane, e8m0_of(ks));             \
     /* the copies of the tile two ahead are issued under the MFMAs of S^T, not in front of them: right */ \
     /* after the barrier their scalar address chain would run in every wave at once with the pipe idle */ \
-    if (i + kAhead < nt) dma(entry(i + kAhead), slot_prev);                                             \
+    if (i + kAhead < t_end) dma(entry(i + kAhead), slot_prev);                                          \
     slot_prev = slot;                                                                                   \
     slot = slot == kRingT - 1 ? 0 : slot + 1;                                                           \
     const float ct = (FP8 && !POW2) ? c * ks : c;                                                       \
     softmax_pv_tile<FP8, STATIC, LEAN, MASKED, POW2>(w, kbuf + kKBytes, ct, tail, lane);                \
   }
-  // Half-tile loop.  Every wave runs the same number of iterations (the longest group's), so the barriers match.
-  // A group's leading full halves take the copy of the code without masking; what is left -- at most the one
-  // partial half at the very end of the keys and one idle iteration of a shorter group -- takes the general copy.
+  // Half-tile loop.  The leading full halves take the copy of the code without masking; the one partial half at the
+  // very end of the keys, if any, takes the general copy.
 #define PKH3_SHORT_LOOP(STATIC, FULL, FROM, TO)                                                         \
   for (int i = FROM; i < TO; ++i) {                                                                     \
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
@@ -627,8 +658,8 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
     }                                                                                                   \
   }
   if constexpr (HALFMODE) {
-    const int n_iter = (n_half + GROUPS - 1) / GROUPS;
-    const int n_lead = max(0, min(n_mine, sk / 32 - h_begin));  // leading full halves of this group
+    const int n_iter = n_half;
+    const int n_lead = sk / 32;  // leading full halves
     if (static_max) {
       PKH3_SHORT_LOOP(true, true, 0, n_lead)
       PKH3_SHORT_LOOP(true, false, n_lead, n_iter)
@@ -638,56 +669,13 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
       PKH3_SHORT_LOOP(false, false, n_lead, n_iter)
       PKH3_MFMA_DRAIN(w);
     }
-    if constexpr (SPLIT) {
-      // Add the groups' partial results into group 0, one group at a time through LDS.  On the bounded-logit
-      // path nothing was subtracted, so numerators and row sums just add; on the running-max path each side
-      // is first brought to the common maximum.
-      __syncthreads();  // every group is done with its ring
-      float* mbuf = (float*)(lds_raw + wq * kMergeBytes);
-#pragma unroll 1
-      for (int src = 1; src < GROUPS; ++src) {
-        if (group == src) {
-#pragma unroll
-          for (int db = 0; db < 8; ++db)
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb) *(f32x4*)(mbuf + ((db * 2 + qb) * 64 + lane) * 4) = w.o[db][qb];
-#pragma unroll
-          for (int qb = 0; qb < 2; ++qb) {
-            mbuf[64 * 64 + qb * 64 + lane] = w.l[qb];
-            mbuf[64 * 64 + 128 + qb * 64 + lane] = w.m[qb];
-          }
-        }
-        __syncthreads();
-        if (group == 0) {
-#pragma unroll
-          for (int qb = 0; qb < 2; ++qb) {
-            const float l2 = mbuf[64 * 64 + qb * 64 + lane], m2 = mbuf[64 * 64 + 128 + qb * 64 + lane];
-            float a1 = 1.0f, a2 = 1.0f;
-            if (!static_max) {
-              const float mn = fmaxf(w.m[qb], m2);
-              a1 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w.m[qb] - mn);
-              a2 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m2 - mn);
-              w.m[qb] = mn;
-            }
-            w.l[qb] = w.l[qb] * a1 + l2 * a2;
-#pragma unroll
-            for (int db = 0; db < 8; ++db) {
-              const f32x4 v4 = *(const f32x4*)(mbuf + ((db * 2 + qb) * 64 + lane) * 4);
-#pragma unroll
-              for (int rr = 0; rr < 4; ++rr) w.o[db][qb][rr] = w.o[db][qb][rr] * a1 + v4[rr] * a2;
-            }
-          }
-        }
-        __syncthreads();
-      }
-    }
   } else if (static_max) {
-    PKH3_TILE_LOOP(true, false, 0, nt - n_masked)
-    PKH3_TILE_LOOP(true, true, nt - n_masked, nt)
+    PKH3_TILE_LOOP(true, false, t_begin, t_end - n_masked)
+    PKH3_TILE_LOOP(true, true, t_end - n_masked, t_end)
     PKH3_MFMA_DRAIN(w);
   } else {
-    PKH3_TILE_LOOP(false, false, 0, nt - n_masked)
-    PKH3_TILE_LOOP(false, true, nt - n_masked, nt)
+    PKH3_TILE_LOOP(false, false, t_begin, t_end - n_masked)
+    PKH3_TILE_LOOP(false, true, t_end - n_masked, t_end)
     PKH3_MFMA_DRAIN(w);
   }
 #undef PKH3_TILE_LOOP
@@ -760,14 +748,67 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   // (16-byte chunks XOR-swizzled by the row so both directions are conflict-free) and stores whole 256-byte rows,
   // 16 bytes per lane.
   __bf16* ob = (__bf16*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
+  __syncthreads();  // every wave is done reading K/V tiles: the LDS becomes staging space
+  if constexpr (PARTS) {
+    if (parts > 1) {
+      // `parts` workgroups hold a share of this unit's result each.  Every wave leaves its partial result in global
+      // scratch and counts itself in; the wave that finds all the others counted adds their partials to its own and
+      // goes on to write the output, the others are done.  Partials and counter move through device-coherent
+      // stores, loads and atomics: a wave counts itself in only after its stores have completed, and reads the
+      // others' partials only after it has seen their counts.
+      const int64_t wslot = kMergeBytes / 4;   // floats per wave
+      float* mine = p.split_scratch + ((int64_t)(part_base + ul * parts + part) * WAVES + wave) * wslot;
+#pragma unroll
+      for (int db = 0; db < 8; ++db)
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) store_device(mine + ((db * 2 + qb) * 64 + lane) * 4, w.o[db][qb]);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        store_device(mine + 64 * 64 + qb * 64 + lane, w.l[qb]);
+        store_device(mine + 64 * 64 + 128 + qb * 64 + lane, w.m[qb]);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      int arrived = 0;
+      if (lane == 0)
+        arrived = __hip_atomic_fetch_add(p.split_cnt + (cnt_base + ul) * WAVES + wave, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      arrived = __builtin_amdgcn_readfirstlane(arrived);
+      if (arrived != parts - 1) return;
+      // The partials are added up in the order of the shares, whichever wave does it (its own comes back from the
+      // scratch like the others), so the result does not depend on which workgroup finished last.
+#pragma unroll 1
+      for (int src = 0; src < parts; ++src) {
+        const float* theirs = p.split_scratch + ((int64_t)(part_base + ul * parts + src) * WAVES + wave) * wslot;
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          const float l2 = load_device(theirs + 64 * 64 + qb * 64 + lane), m2 = load_device(theirs + 64 * 64 + 128 + qb * 64 + lane);
+          // On the bounded-logit path nothing was subtracted, so numerators and row sums just add; on the
+          // running-max path each side is first brought to the common maximum.  Share 0 starts the sum.
+          float a1 = src == 0 ? 0.0f : 1.0f, a2 = 1.0f;
+          if (!static_max && src != 0) {
+            const float mn = fmaxf(w.m[qb], m2);
+            a1 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w.m[qb] - mn);
+            a2 = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m2 - mn);
+            w.m[qb] = mn;
+          } else if (src == 0) {
+            w.m[qb] = m2;
+          }
+          w.l[qb] = src == 0 ? l2 : w.l[qb] * a1 + l2 * a2;
+#pragma unroll
+          for (int db = 0; db < 8; ++db) {
+            const f32x4 v4 = load_device4(theirs + ((db * 2 + qb) * 64 + lane) * 4);
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) w.o[db][qb][rr] = src == 0 ? v4[rr] : w.o[db][qb][rr] * a1 + v4[rr] * a2;
+          }
+        }
+      }
+    }
+  }
   float inv[2];
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {
     const float lt = wave_sum_groups(w.l[qb]);
     inv[qb] = lt > 0.f ? 1.0f / lt : 0.f;
   }
-  __syncthreads();  // every wave is done reading K/V tiles (SPLIT: and merge buffers): the LDS becomes staging space
-  if (SPLIT && group != 0) return;  // the merged result lives in group 0
   char* stage = lds_raw + wq * kStageBytes;
   {
     const int c16 = lane & 15, g = lane >> 4;
@@ -812,31 +853,99 @@ __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : WAVES == kShortWa
   }
 }
 
-template <bool FP8, bool POW2, bool SPARSE, int WAVES, bool SPLIT = false>
-static void launch_variant(FwdParams p, int unit0, int units, hipStream_t st) {
-  p.unit0 = unit0;
-  p.units = units;
-  hipLaunchKernelGGL((attn_fwd_kernel<FP8, SPARSE, WAVES, SPLIT, POW2>), dim3((units + 7) / 8 * 8), dim3(64 * WAVES), 0, st, p);
+// The block-sparse kernel and the short-key dense kernel.
+template <bool FP8, bool SPARSE, int WAVES, bool POW2>
+__global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : 3)) void attn_fwd_kernel(FwdParams p) {
+  __shared__ __attribute__((aligned(1024))) char lds_raw[fwd_lds_bytes<FP8, SPARSE, WAVES>()];
+  attn_fwd_body<FP8, SPARSE, WAVES, POW2>(p, blockIdx.x, 0, p.sec_units[0], 1, 0, 0, lds_raw);
+}
+
+// The long dense kernel: a launch of up to kSections sections, handed out in this order as CUs fall free.  Section 0
+// holds whole units (one workgroup each); the later ones the units of a thinly filled last round, each shared out
+// among sec_parts[] workgroups.
+template <bool FP8, bool POW2>
+__global__ __launch_bounds__(64 * kDenseWaves, 1) void attn_fwd_dense_kernel(FwdParams p) {
+  __shared__ __attribute__((aligned(1024))) char lds_raw[fwd_lds_bytes<FP8, false, kDenseWaves>()];
+  static_assert(kSections == 3, "the section look-up below is written out for three");
+  const int bid = blockIdx.x, b0 = p.sec_blocks[0], b1 = p.sec_blocks[1];
+  const int sec = (bid >= b0 ? 1 : 0) + (bid >= b0 + b1 ? 1 : 0);
+  const int blk = bid - (sec >= 1 ? b0 : 0) - (sec >= 2 ? b1 : 0);
+  const int unit0 = (sec >= 1 ? p.sec_units[0] : 0) + (sec >= 2 ? p.sec_units[1] : 0);
+  const int units = sec == 0 ? p.sec_units[0] : sec == 1 ? p.sec_units[1] : p.sec_units[2];
+  const int parts = sec == 0 ? p.sec_parts[0] : sec == 1 ? p.sec_parts[1] : p.sec_parts[2];
+  // partial results and counters of section 2 lie behind those of section 1 (section 0 has none)
+  const bool behind = sec == 2 && p.sec_parts[1] > 1;
+  const int part_base = behind ? p.sec_units[1] * p.sec_parts[1] : 0, cnt_base = behind ? p.sec_units[1] : 0;
+  attn_fwd_body<FP8, false, kDenseWaves, POW2>(p, blk, unit0, units, parts, part_base, cnt_base, lds_raw);
+}
+
+static int blocks_of(int workgroups) { return (workgroups + 7) / 8 * 8; }
+
+// How a long dense call ends.  One 12-wave workgroup per CU at a time: the call runs in rounds of `cus` workgroups, and
+// `rest` units left for a last round leave CUs idle for a whole workgroup's duration.  Sharing each of those units out
+// among P workgroups (1/P of the key tiles each) gives workgroups of 1/P of the duration that again run in rounds of
+// `cus`; one or two such sections (P1 for the units that fill a round, P2 for what is left) end the call in
+// 1/P1 + 1/P2 of a whole round.  The cheapest plan within the scratch (one partial result per workgroup) is taken.
+struct TailPlan {
+  int units[2], parts[2];
+};
+static TailPlan plan_tail(int rest, int cus, int n_tiles, int64_t max_workgroups) {
+  TailPlan best{{rest, 0}, {1, 1}};
+  if (rest <= 0 || cus <= 0) return best;
+  const int pmax = max(1, min(kMaxParts, n_tiles / kMinPartTiles));
+  double best_cost = 1.0;
+  auto consider = [&](int u1, int p1, int u2, int p2) {
+    const int64_t wgs = (p1 > 1 ? (int64_t)u1 * p1 : 0) + (p2 > 1 ? (int64_t)u2 * p2 : 0);
+    if (wgs > max_workgroups) return;
+    const double cost = 1.0 / p1 + (u2 > 0 ? 1.0 / p2 : 0.0);
+    if (cost < best_cost - 1e-9) best_cost = cost, best = TailPlan{{u1, u2}, {p1, p2}};
+  };
+  const int p_all = min(pmax, cus / rest);     // every unit of the rest in one round of workgroups
+  if (p_all > 1) consider(rest, p_all, 0, 1);
+  for (int p1 = 2; p1 <= pmax; ++p1) {
+    const int u1 = cus / p1;                   // units that fill one round at p1
+    if (u1 <= 0 || u1 >= rest) continue;
+    const int p2 = min(pmax, cus / (rest - u1));
+    if (p2 >= 1) consider(u1, p1, rest - u1, p2);
+  }
+  return best;
 }
 
 template <bool FP8, bool POW2 = false>
-static void launch_fp(const FwdParams& p, int cus, hipStream_t st) {
+static hipError_t launch_fp(FwdParams p, int cus, hipStream_t st) {
   const int nQ32 = p.nQ64 * 2;
   auto units = [&](int blocks) { return p.B * p.H * ((nQ32 + blocks - 1) / blocks); };
-  if (p.plan) return launch_variant<FP8, POW2, true, kSparseWaves>(p, 0, units(kSparseWaves), st);
-  if (p.nKt <= kShortMaxTiles && !p.long_key_kernel) return launch_variant<FP8, POW2, false, kShortWaves>(p, 0, units(kShortWaves), st);
-  // Long dense call: one workgroup per CU at a time, so the call runs in rounds of `cus` workgroups.  When the
-  // last round would be less than two thirds full, its query tiles go to the SPLIT form instead (three
-  // workgroups of a third of the duration each per tile), launched behind the whole rounds.
+  for (int i = 0; i < kSections; ++i) p.sec_units[i] = p.sec_blocks[i] = 0, p.sec_parts[i] = 1;
+  if (p.plan) {
+    p.sec_units[0] = units(kSparseWaves);
+    hipLaunchKernelGGL((attn_fwd_kernel<FP8, true, kSparseWaves, POW2>), dim3(blocks_of(p.sec_units[0])), dim3(64 * kSparseWaves), 0, st, p);
+    return hipGetLastError();
+  }
+  if (p.nKt <= kShortMaxTiles && !p.long_key_kernel) {
+    p.sec_units[0] = units(kShortWaves);
+    hipLaunchKernelGGL((attn_fwd_kernel<FP8, false, kShortWaves, POW2>), dim3(blocks_of(p.sec_units[0])), dim3(64 * kShortWaves), 0, st, p);
+    return hipGetLastError();
+  }
   const int n = units(kDenseWaves);
   const int whole = cus > 0 ? n / cus * cus : n, rest = n - whole;
-  constexpr int kGroups = kDenseWaves / kShortWaves;
-  if (whole > 0 && rest > 0 && rest * kGroups <= 2 * cus && !p.long_key_kernel) {
-    launch_variant<FP8, POW2, false, kDenseWaves>(p, 0, whole, st);
-    launch_variant<FP8, POW2, false, kDenseWaves, true>(p, whole * kGroups, rest * kGroups, st);
-  } else {
-    launch_variant<FP8, POW2, false, kDenseWaves>(p, 0, n, st);
+  p.sec_units[0] = n;
+  if (whole > 0 && rest > 0 && !p.long_key_kernel && p.split_cnt) {
+    const int64_t cap = (int64_t)(p.split_scratch_bytes / ((size_t)kDenseWaves * kMergeBytes));
+    const TailPlan t = plan_tail(rest, cus, p.nKt, cap);
+    if (t.parts[0] > 1 || t.parts[1] > 1) {
+      p.sec_units[0] = whole;
+      p.sec_units[1] = t.units[0], p.sec_parts[1] = t.parts[0];
+      p.sec_units[2] = t.units[1], p.sec_parts[2] = t.parts[1];
+      // the arrival counters of the shared units start at zero
+      const int shared = (t.parts[0] > 1 ? t.units[0] : 0) + (t.parts[1] > 1 ? t.units[1] : 0);
+      hipError_t e = launch_fill_zero((unsigned*)p.split_cnt, shared * kDenseWaves, st);
+      if (e != hipSuccess) return e;
+    }
   }
+  int blocks = 0;
+  for (int i = 0; i < kSections; ++i) blocks += p.sec_blocks[i] = blocks_of(p.sec_units[i] * p.sec_parts[i]);
+  hipLaunchKernelGGL((attn_fwd_dense_kernel<FP8, POW2>), dim3(blocks), dim3(64 * kDenseWaves), 0, st, p);
+  return hipGetLastError();
 }
 
 // CUs of the current device, asked once per device; threads that race here store the same value
@@ -862,10 +971,9 @@ hipError_t launch_attn_fwd(const FwdParams& p, hipStream_t st) {
   int cus = 0;
   hipError_t e = device_cu_count(&cus);
   if (e != hipSuccess) return e;
-  if (p.fp8 && p.fp8_pow2) launch_fp<true, true>(p, cus, st);
-  else if (p.fp8) launch_fp<true>(p, cus, st);
-  else launch_fp<false>(p, cus, st);
-  return hipGetLastError();
+  if (p.fp8 && p.fp8_pow2) return launch_fp<true, true>(p, cus, st);
+  if (p.fp8) return launch_fp<true>(p, cus, st);
+  return launch_fp<false>(p, cus, st);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -13,12 +13,21 @@ namespace pkh3 {
 constexpr int kSparseRows = 4;
 constexpr int kSparseLists = 1 + kSparseRows;
 
+// Long dense calls may end on workgroups that share a unit's key tiles and merge their partial results through global
+// scratch: one wave's partial result (O^T 128 x 32, row sums, row maxima, fp32), and the most such workgroups a call
+// is planned with (two rounds of workgroups on a 256-CU part; a call that would need more ends on whole workgroups).
+constexpr int kPartialBytes = 64 * 64 * 4 + 4 * 64 * 4;
+constexpr int kMaxPartWorkgroups = 512;
+constexpr int kSections = 3;     // sections of a long dense launch
+constexpr int kShortMaxTiles = 16;  // dense calls with at most this many key tiles run the short-key kernel
+
 // Where each intermediate lives inside the caller's workspace (byte offsets, 256-aligned).
 struct WsPlan {
   int nQ64;      // 64-query blocks, padded to a multiple of 4 (one workgroup = 4 waves x 64 queries)
   int nKt;       // 64-key tiles
   int kvTileBytes;  // bytes of one [K tile | V tile] record
-  size_t kv_off, kscale_off, cnt_off, idx_off, plan_off, plan_cnt_off, kmax_off, total;
+  size_t kv_off, kscale_off, cnt_off, idx_off, plan_off, plan_cnt_off, kmax_off, split_off, split_cnt_off, total;
+  size_t split_bytes;  // bytes at split_off: partial results of the long dense form's paired workgroups
 };
 
 // One side (Q or K) of the normalise + rotate + lay-out pass.
@@ -81,8 +90,16 @@ struct FwdParams {
   const float* kmax;        // [B*H] largest K' row norm
   int fp8;
   int fp8_pow2;         // fp8: the block scales are powers of two and ride in the scaled MFMA's operands
-  int long_key_kernel;  // only the plain long-key form (no short-key form, no split last round)
-  int unit0, units;     // filled per launch: the workgroup units [unit0, unit0 + units) this launch covers
+  int long_key_kernel;  // only the plain long-key form (no short-key form, no shared last round)
+  // scratch of the long dense form's shared units (see launch_fp): partial results, and arrival counters (one per
+  // wave of a unit of the call's last round)
+  float* split_scratch;
+  size_t split_scratch_bytes;
+  int* split_cnt;
+  // filled per launch: the sections of the launch.  A unit is one workgroup's block of queries; section i covers
+  // sec_units[i] units after those of the sections before it, sec_parts[i] workgroups per unit, in sec_blocks[i]
+  // workgroup indices (a multiple of 8)
+  int sec_units[kSections], sec_parts[kSections], sec_blocks[kSections];
 };
 
 // ---- projection GEMMs (pkh3_gemm.hip) -------------------------------------------------------------------

@@ -26,7 +26,7 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from .layout import audio_position_ids, video_position_ids
+from .layout import TILE, audio_position_ids, video_position_ids
 
 PATCH_SIZE = (1, 2, 2)         # transformer patch (t, h, w)          -- geometry.py:26
 VIDEO_LATENT_CHANNELS = 24     #                                       -- geometry.py:22
@@ -300,6 +300,45 @@ def row_timesteps(layout: PackedLayout, *, video_t: float, audio_t: float, condi
         raise ValueError("layout rows are not covered by its index sets")
     unique, index = torch.unique(t, sorted=True, return_inverse=True)
     return unique.to(torch.float32), index.to(torch.int32)
+
+
+def packed_window_tile_map(layout: PackedLayout, *, window_frames: int = 2, global_fraction: float = 0.10,
+                           seed: int = 0) -> torch.Tensor:
+    """bool ``[ceil(S/64), ceil(S/64)]`` map of the 64x64 tiles a local spatio-temporal window keeps on a PACKED
+    document (text, condition rows, audio, video in one sequence: src/pika_h3/core/wrapper.py:192-204,
+    src/pika_h3/core/geometry.py:83-92), the counterpart of ``layout.local_window_tile_map`` for a bare video grid.
+
+    Text rows, condition rows (keyframes, references) and audio rows attend, and are attended, globally: a tile
+    that holds any such row is kept whole, as a query tile and as a key tile -- which also settles the tiles that
+    straddle two segments.  Two tiles of target video rows are kept when the latent frames they cover, read from
+    ``layout.position_ids[:, 0]``, lie at most ``window_frames`` apart, or when a seeded draw makes the pair one of
+    the ``global_fraction`` random global tiles.  The diagonal is always kept."""
+    if not 0.0 <= global_fraction <= 1.0:
+        raise ValueError("global_fraction must be in [0, 1]")
+    if window_frames < 0:
+        raise ValueError("window_frames must be >= 0")
+    S = layout.sequence_length
+    nt = (S + TILE - 1) // TILE
+    is_video = torch.zeros(S, dtype=torch.bool)
+    is_video[layout.video_indices.cpu()[layout.num_condition_video_rows:]] = True
+    frame = torch.floor(layout.position_ids[:, 0].detach().to("cpu", torch.float64)).to(torch.int64)
+    pad = nt * TILE - S
+    vid = torch.cat([is_video, torch.zeros(pad, dtype=torch.bool)]).view(nt, TILE)
+    other = torch.cat([~is_video, torch.zeros(pad, dtype=torch.bool)]).view(nt, TILE)    # padding rows belong to nobody
+    fr = torch.cat([frame, torch.zeros(pad, dtype=torch.int64)]).view(nt, TILE)
+    big = torch.iinfo(torch.int64).max
+    lo = torch.where(vid, fr, torch.full_like(fr, big)).amin(dim=1)
+    hi = torch.where(vid, fr, torch.full_like(fr, -big)).amax(dim=1)
+    everywhere = other.any(dim=1)                    # tiles with a text / condition / audio row
+    only_video = ~everywhere
+    gap = torch.maximum(lo[None, :] - hi[:, None], lo[:, None] - hi[None, :])   # frames between the two ranges
+    keep = (gap <= window_frames) & only_video[:, None] & only_video[None, :]
+    keep |= everywhere[:, None] | everywhere[None, :]
+    if global_fraction > 0.0:
+        g = torch.Generator().manual_seed(int(seed))
+        keep |= torch.rand((nt, nt), generator=g) < global_fraction
+    keep |= torch.eye(nt, dtype=torch.bool)
+    return keep
 
 
 class LayoutCache:

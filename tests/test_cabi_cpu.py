@@ -290,6 +290,14 @@ def test_kv_prepare_argument_errors(lib):
     assert lib.pkh3_workspace_bytes(C.byref(a)) == dense
     a.blk_row_ptr, a.blk_col_idx = 0x20000, 0x30000
     assert lib.pkh3_workspace_bytes(C.byref(a)) > dense
+    # long dense calls: behind the K/V side, a bounded scratch for the workgroup pairs that may end the call
+    a = _valid_args(); a.Sk = 4096; a.H = 24
+    a.Sq = 384
+    small = lib.pkh3_workspace_bytes(C.byref(a))
+    a.Sq = 48360
+    big = lib.pkh3_workspace_bytes(C.byref(a))
+    a.Sq = 1 << 20
+    assert 0 < big - small <= 512 * 12 * 17408 + 512 * 48 + 512 and lib.pkh3_workspace_bytes(C.byref(a)) == big
 
 
 def test_out_proj_argument_errors(lib):

@@ -266,7 +266,7 @@ def test_joint_and_cross_full_tensor():
     from pika_h3_flex_amd import workloads
 
     joint = workloads.make("joint", seed=1, device="cuda")
-    out, _, _ = _run(joint)  # 3,120 query tiles: whole rounds in the 12-wave form, the last 48 in the split form
+    out, _, _ = _run(joint)  # 3,120 query tiles: 12 whole rounds, the last 48 tiles shared out five ways each
     _check_full(out, _oracle_full(joint), label="joint video+audio")
     mass = _indicator_mass(joint)
     assert float((mass - 1.0).abs().max()) < 1.5e-2
@@ -526,16 +526,59 @@ def test_processor_on_a_packed_document():
     assert float((y.float() - yref.float()).abs().max()) < 3e-2
 
 
+@pytest.mark.parametrize("fp8", [False, True, "pow2"])
+def test_processor_block_sparse_on_a_packed_document(fp8):
+    """The block-sparse and fp8 kernels pointed at a packed document (text, first and last keyframe, audio, video):
+    the processor with the map ``packing.packed_window_tile_map`` makes of the layout, against the oracle with
+    the same map expanded to elements.  Text, keyframe and audio rows attend globally, video rows within a window
+    of one latent frame plus seeded random tiles."""
+    import pika_h3_flex_amd as pk
+    from pika_h3_flex_amd import packing as P
+    from oracle import attention_oracle as O
+
+    torch.manual_seed(5)
+    H, hidden = 2, 256
+    lay = P.build_layout(num_text_tokens=37, num_latent_frames=9, latent_height=16, latent_width=24, num_audio_latents=21,
+                         keyframe_anchors=("first", "last"))
+    S = lay.sequence_length
+    tm = P.packed_window_tile_map(lay, window_frames=1, global_fraction=0.05, seed=2)
+    assert 0.3 < float(tm.float().mean()) < 0.9          # a real mixture of kept and dropped tiles
+    x = (torch.randn(1, S, hidden) * 0.5).cuda().to(torch.bfloat16)
+    attn = _Attn(hidden, H).cuda().to(torch.bfloat16)
+    proc = pk.PikaH3AttnProcessor()
+    bm = pk.BlockMask.from_dense(tm, device="cuda")
+    with torch.no_grad():
+        y = proc(attn, x, position_ids=lay.position_ids.cuda(), block_mask=bm, fp8_qk=fp8)
+        dense = proc(attn, x, position_ids=lay.position_ids.cuda(), fp8_qk=fp8)
+        q, k, v = (f(x).view(1, S, H, 128) for f in (attn.to_q, attn.to_k, attn.to_v))
+        ref = O.reference_layer(q.cpu(), k.cpu(), v.cpu(), q_norm_weight=attn.norm_q.weight.float().cpu(),
+                                k_norm_weight=attn.norm_k.weight.float().cpu(), rope_q=O.rope_tables(lay.position_ids),
+                                rope_mode=O.ROPE_INTERLEAVED, tile_map=tm, fp8_qk=fp8)
+        yref = attn.to_out[0](ref.to(torch.bfloat16).view(1, S, hidden).cuda())
+    err, cos = O.max_abs_and_cosine(y.cpu(), yref.cpu())
+    print(f"packed document, block map density {float(tm.float().mean()):.3f}, fp8={fp8}: max_abs={err:.3e} cos={cos:.7f}", flush=True)
+    assert cos >= (0.995 if fp8 else 0.9999) and err < 3e-2
+    # the map changes the result: rows of the video segment lose keys the dense call sees
+    assert float((y.float() - dense.float()).abs().max()) > 1e-3
+    # rows that attend globally (text, keyframes, audio: everything before the target video rows) keep every key
+    n_global = S - lay.counts.video
+    full_rows = (n_global // 64) * 64
+    assert float((y[:, :full_rows].float() - dense[:, :full_rows].float()).abs().max()) <= 4e-3
+
+
+@pytest.mark.parametrize("S", [4200, 4600])
 @pytest.mark.parametrize("variant", ["bf16", "bf16_large_logits", "fp8", "key_mask"])
-def test_split_last_round_form(variant):
-    """A long dense call whose last round of workgroups is thinly filled hands those query tiles to the form
-    that splits the keys three ways inside the workgroup (H=24, S=4200: 264 query tiles on a 256-CU part, the
-    last 8 go there).  Its results must agree with the plain long-key form on the same inputs and with the
-    oracle on sampled rows of the last head, where those tiles are."""
+def test_shared_last_round(variant, S):
+    """A long dense call whose last round of workgroups is thinly filled shares each of those query tiles out among
+    several workgroups (a slice of the key tiles each) that merge their partial results through the workspace.
+    H=24 on a 256-CU part: S=4200 makes 264 query tiles, the last 8 shared two ways; S=4600 makes 288, the last 32
+    shared three ways.  The results must agree with the plain long-key form on the same inputs and with the oracle
+    on sampled rows of the last head, where those tiles are, and must not depend on which workgroup finishes last:
+    repeated calls give the same bits."""
     import pika_h3_flex_amd as pk
     from oracle import attention_oracle as O
 
-    B, S, H = 1, 4200, 24
+    B, H = 1, 24
     gen = torch.Generator().manual_seed(404)
     q, k, v = ((torch.randn((B, S, H, D), generator=gen)).to(torch.bfloat16) for _ in range(3))
     wq = torch.ones(D) * (4.0 if variant == "bf16_large_logits" else 1.0)
@@ -554,18 +597,20 @@ def test_split_last_round_form(variant):
     qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
     out = pk.attention(qc, kc, vc, **opts)
     plain = pk.attention(qc, kc, vc, long_key_kernel=True, **opts)
+    again = [pk.attention(qc, kc, vc, **opts) for _ in range(3)]
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all()
+    assert all(torch.equal(out, a) for a in again)
     err, cos = O.max_abs_and_cosine(out.cpu(), plain.cpu())
-    print(f"split vs plain long form [{variant}]: max_abs={err:.3e} cos={cos:.8f}", flush=True)
+    print(f"shared last round vs plain long form [{variant}, S={S}]: max_abs={err:.3e} cos={cos:.8f}", flush=True)
     # outputs of peaked softmaxes reach |O| ~ 3, where one bf16 step is 1.6e-2
     assert err <= (2e-2 if variant == "bf16_large_logits" else 8e-3) and cos >= 0.99999
-    rows = torch.tensor(sorted({0, 383, 384, 1151, 1152, 1535, 1536, 2000, 3071, 3072, 3500, 4095, 4096, 4199}))
+    rows = torch.tensor(sorted({0, 383, 384, 1151, 1152, 1535, 1536, 2000, 3071, 3072, 3500, 4095, 4096, S - 1}))
     hs = torch.tensor([22, 23])
     ref = O.reference_layer(q[:, :, hs], k[:, :, hs], v[:, :, hs], q_rows=rows, **ref_opts)
     got = out[:, rows.cuda()][:, :, hs.cuda()].cpu()
     err, cos = O.max_abs_and_cosine(got, ref)
-    print(f"split vs oracle [{variant}]: max_abs={err:.3e} cos={cos:.7f}", flush=True)
+    print(f"shared last round vs oracle [{variant}, S={S}]: max_abs={err:.3e} cos={cos:.7f}", flush=True)
     if variant == "fp8":
         assert cos >= 0.995
     else:

@@ -307,7 +307,7 @@ def test_same_logits_through_both_softmax_forms():
         assert e12 <= 8e-3 and c12 >= 0.99999
 
 
-@pytest.mark.parametrize("variant", ["dense_rope_mask", "sparse_fp8", "long_dense_split_last_round"])
+@pytest.mark.parametrize("variant", ["dense_rope_mask", "sparse_fp8", "long_dense_shared_last_round"])
 def test_hip_graph_replays_match_eager(variant):
     """The layer call allocates nothing and only launches kernels on the caller's stream, so it can be captured
     into a HIP graph.  Every replay, with fresh inputs in the captured buffers and eager work in between, must
@@ -315,8 +315,8 @@ def test_hip_graph_replays_match_eager(variant):
     import pika_h3_flex_amd as pk
 
     B, S, H, D = 1, 333, 2, 128
-    if variant == "long_dense_split_last_round":
-        S, H = 4200, 24  # 264 query tiles on a 256-CU part: two launches (whole rounds, then the split form)
+    if variant == "long_dense_shared_last_round":
+        S, H = 4200, 24  # 264 query tiles on a 256-CU part: the counter fill, then one launch whose last 8 tiles are shared two ways
     gen = torch.Generator().manual_seed(91)
     dev = "cuda"
     q, k, v = (_rand((B, S, H, D), gen).to(dev) for _ in range(3))
@@ -327,7 +327,7 @@ def test_hip_graph_replays_match_eager(variant):
         cos, sin = pk.rope_tables(pos.to(dev))
         mask = (torch.rand((B, S), generator=gen) < 0.7).to(dev)
         opts.update(rope_mode=1, rope_q=(cos, sin), key_mask=mask)
-    elif variant == "long_dense_split_last_round":
+    elif variant == "long_dense_shared_last_round":
         pass
     else:
         tm = torch.rand((6, 6), generator=gen) < 0.5

@@ -410,10 +410,10 @@ def test_document_kwargs_drive_the_fused_block():
 
 
 @pytest.mark.parametrize("S,H,variant", [(300, 2, "dense"), (1000, 3, "fp8"), (777, 2, "sparse"), (130, 1, "short"),
-                                         (4200, 24, "split"), (4200, 24, "split_fp8")])
+                                         (4200, 24, "shared"), (4200, 24, "shared_fp8")])
 def test_attention_writes_the_out_projection_images(S, H, variant):
     """With PKH3_FLAG_O_IMAGES the attention epilogue writes what pkh3_pack_rows would make of its row-major output:
-    the same bytes for every image row that exists, in every form of the kernel (long, short-key, split, block-sparse)."""
+    the same bytes for every image row that exists, in every form of the kernel (long, short-key, shared last round, block-sparse)."""
     import pika_h3_flex_amd as pk
     from pika_h3_flex_amd import projections as P
 
@@ -422,9 +422,9 @@ def test_attention_writes_the_out_projection_images(S, H, variant):
     w = (1.0 + 0.1 * torch.randn(128, generator=g)).cuda()
     pos = (torch.rand((S, 3), generator=g, dtype=torch.float64) * 20).cuda()
     opts = dict(q_norm_weight=w, k_norm_weight=w, rope_mode=pk.ROPE_INTERLEAVED, rope_q=pk.rope_tables(pos))
-    if variant in ("fp8", "split_fp8"):
+    if variant in ("fp8", "shared_fp8"):
         opts["fp8_qk"] = True
-    # "split": 264 query tiles on a 256-CU part: whole rounds in the 12-wave form, the last 8 tiles in the split form
+    # "shared": 264 query tiles on a 256-CU part: whole rounds, then the last 8 tiles shared out two ways
     if variant == "sparse":
         nt = (S + 63) // 64
         keep = torch.rand((nt, nt), generator=g) < 0.5
