@@ -182,9 +182,12 @@ def bench_block(args, pk, workloads, dev) -> dict:
     return line
 
 
-ATTENTION_WORKLOADS = ("plumbing", "480p", "768p", "joint", "cross", "480p-sparse", "480p-sparse-fp8", "480p-fp8")
-# what the default run measures beside the headline (same process, after the headline's timed region)
-OTHER_WORKLOADS = ("480p-fp8", "480p-sparse", "480p-sparse-fp8", "768p", "joint", "cross", "480p-block")
+ATTENTION_WORKLOADS = ("plumbing", "480p", "768p", "joint", "cross", "480p-sparse", "480p-sparse-fp8", "480p-fp8",
+                       "480p-fp8-pow2", "480p-sparse-fp8-pow2")
+# what the default run measures beside the headline (same process, after the headline's timed region); "-pow2" is the
+# opt-in fp8 rule with power-of-two block scales applied by the scaled MFMA (PKH3_FLAG_FP8_POW2_SCALES)
+OTHER_WORKLOADS = ("480p-fp8", "480p-fp8-pow2", "480p-sparse", "480p-sparse-fp8", "480p-sparse-fp8-pow2", "768p", "joint",
+                   "cross", "480p-block")
 
 
 def algorithmic_bytes(B, Sq, Sk, H, D, fp8, density=1.0):
@@ -215,13 +218,14 @@ class AttentionCase:
         if inp.key_mask is not None:
             opts.update(key_mask=inp.key_mask)
         self.density = 1.0
-        self.fp8 = name.endswith("fp8")
+        self.fp8 = "fp8" in name.split("-")
+        self.pow2 = name.endswith("-pow2")
         if "sparse" in name:
             tm = pk.local_window_tile_map(self.Sq, inp.tokens_per_frame, window_frames=2, global_fraction=0.10, seed=seed)
             self.density = float(tm.float().mean())
             opts.update(block_mask=pk.BlockMask.from_dense(tm, device=dev))
         if self.fp8:
-            opts.update(fp8_qk=True)
+            opts.update(fp8_qk="pow2" if self.pow2 else True)
         self.opts = opts
         self.flops = inp.flops * self.density
         self.out = torch.empty_like(inp.q)
@@ -233,7 +237,13 @@ class AttentionCase:
 
     def describe(self):
         return (f"{self.name} attention layer: B={self.B}, H={self.H}, D={self.D}, Sq={self.Sq}, Sk={self.Sk}, "
-                f"QK-RMSNorm + 3-axis RoPE, non-causal" + (f", block-sparse density {self.density:.3f}" if self.density < 1 else ""))
+                f"QK-RMSNorm + 3-axis RoPE, non-causal" + (f", block-sparse density {self.density:.3f}" if self.density < 1 else "")
+                + (", power-of-two fp8 block scales" if self.pow2 else ""))
+
+    def kernel_name(self):
+        if self.density < 1:
+            return "attn_fwd_kernel (block-sparse, 8 waves)"
+        return "attn_fwd_kernel (short-key, 4 waves)" if self.Sk <= 1024 else "attn_fwd_dense_kernel (12 waves)"
 
     def roofline(self, kernel_iters):
         """The attention kernel alone (HIP events on its stream, inside the library) against its MFMA peak, beside
@@ -247,7 +257,7 @@ class AttentionCase:
         r = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
              "frac": round(achieved / peak, 4), "traffic": traffic, "traffic_source": source,
              "algorithmic_bytes": alg, "traffic_over_algorithmic": None if traffic is None else round(traffic / alg, 2),
-             "kernel": "attn_fwd_kernel", "kernel_ms": round(kernel_ms, 4), "flops_per_launch": self.flops}
+             "kernel": self.kernel_name(), "kernel_ms": round(kernel_ms, 4), "flops_per_launch": self.flops}
         if traffic is not None:
             # the other roof: bytes that crossed the L2 boundary per launch (profiled) over this run's kernel time
             rate = traffic / (kernel_ms * 1e-3) / 1e9

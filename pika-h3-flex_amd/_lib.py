@@ -42,7 +42,6 @@ EXPORTS = (
     "pkh3_version",
     "pkh3_strerror",
     "pkh3_last_error",
-    "pkh3_attn_time_kernel",
     "pkh3_packed_bytes",
     "pkh3_pack_weight",
     "pkh3_pack_rows",
@@ -139,8 +138,6 @@ def load() -> C.CDLL:
     lib.pkh3_attn_fwd_noalloc.restype = C.c_int
     lib.pkh3_noalloc_init.argtypes = []
     lib.pkh3_noalloc_init.restype = C.c_int
-    lib.pkh3_attn_time_kernel.argtypes = [C.POINTER(AttnArgs), C.c_void_p, C.c_int, C.POINTER(C.c_float)]
-    lib.pkh3_attn_time_kernel.restype = C.c_int
     lib.pkh3_rope_tables.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_int32), C.c_double, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.pkh3_rope_tables.restype = C.c_int
     lib.pkh3_packed_bytes.argtypes = [C.c_int32, C.c_int32]
@@ -163,6 +160,28 @@ def load() -> C.CDLL:
     lib.pkh3_last_error.argtypes = []
     lib.pkh3_last_error.restype = C.c_char_p
     _lib = lib
+    return lib
+
+
+BENCH_LIB_PATH = os.path.join(os.path.dirname(LIB_PATH), "libpkh3attn_bench.so")
+BENCH_EXPORTS = ("pkh3_attn_time_kernel",)   # include/pkh3_attn_bench.h
+_bench = None
+
+
+def load_bench() -> C.CDLL:
+    """The measurement library (``libpkh3attn_bench.so``, the one call that synchronises with the device): for
+    benchmark harnesses only, never loaded by the product path.  It links against the product library, which is
+    loaded first so that both share one copy of it."""
+    global _bench
+    if _bench is not None:
+        return _bench
+    load()
+    if not os.path.exists(BENCH_LIB_PATH):
+        raise ImportError(f"{BENCH_LIB_PATH} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}`")
+    lib = C.CDLL(BENCH_LIB_PATH)
+    lib.pkh3_attn_time_kernel.argtypes = [C.POINTER(AttnArgs), C.c_void_p, C.c_int, C.POINTER(C.c_float)]
+    lib.pkh3_attn_time_kernel.restype = C.c_int
+    _bench = lib
     return lib
 
 

@@ -1,7 +1,6 @@
 // C ABI of libpkh3attn.so: argument validation (host only, before any HIP call), workspace
 // planning, and the sequence of launches that makes up one attention call.
 #include "../../include/pkh3_attn.h"
-#include "../../include/pkh3_attn_bench.h"
 
 #include <math.h>
 
@@ -283,6 +282,28 @@ int static_scratch(void** out) {
 
 }  // namespace
 
+namespace pkh3 {
+
+// Everything of an attention call except the attention launch itself: validation, workspace planning and the
+// prologue kernels; `out` receives the parameters the attention launch takes.  For the measurement library
+// (pkh3_bench.hip), which times that launch alone.
+int prepare_call(const pkh3_attn_args* a, hipStream_t st, FwdParams* out) {
+  int rc = validate(a, true);
+  if (rc) return rc;
+  Launch L;
+  build(a, a->workspace, L);
+  if (a->workspace_bytes < L.w.total)
+    return fail(PKH3_EWORKSPACE, "workspace too small: %zu < %zu bytes", a->workspace_bytes, L.w.total);
+  if ((rc = run_prologue(a, L, st))) return rc;
+  *out = L.f;
+  g_err[0] = 0;
+  return PKH3_OK;
+}
+
+int report_error(int code, const char* text) { return fail(code, "%s", text); }
+
+}  // namespace pkh3
+
 extern "C" {
 
 int pkh3_version(void) { return PKH3_VERSION; }
@@ -370,39 +391,6 @@ int pkh3_attn_fwd_noalloc(const pkh3_attn_args* a, void* stream) {
   if ((rc = run_prologue(a, L, st))) return rc;
   hipError_t e = launch_attn_fwd(L.f, st);
   if (e != hipSuccess) return hip_fail(e, "attn_fwd");
-  g_err[0] = 0;
-  return PKH3_OK;
-}
-
-int pkh3_attn_time_kernel(const pkh3_attn_args* a, void* stream, int iters, float* ms_out) {
-  if (!ms_out) return fail(PKH3_ENULL, "ms_out is NULL");
-  if (iters < 1) return fail(PKH3_EARG, "iters must be >= 1");
-  int rc = validate(a, true);
-  if (rc) return rc;
-  Launch L;
-  build(a, a->workspace, L);
-  if (a->workspace_bytes < L.w.total)
-    return fail(PKH3_EWORKSPACE, "workspace too small: %zu < %zu bytes", a->workspace_bytes, L.w.total);
-  hipStream_t st = (hipStream_t)stream;
-  if ((rc = run_prologue(a, L, st))) return rc;
-  hipError_t e;
-  if ((e = launch_attn_fwd(L.f, st)) != hipSuccess) return hip_fail(e, "attn_fwd");  // warm
-  hipEvent_t e0, e1;
-  if ((e = hipEventCreate(&e0)) != hipSuccess) return hip_fail(e, "hipEventCreate");
-  if ((e = hipEventCreate(&e1)) != hipSuccess) { hipEventDestroy(e0); return hip_fail(e, "hipEventCreate"); }
-  hipEventRecord(e0, st);
-  for (int i = 0; i < iters; ++i) {
-    if ((e = launch_attn_fwd(L.f, st)) != hipSuccess) break;
-  }
-  hipEventRecord(e1, st);
-  hipError_t es = hipEventSynchronize(e1);
-  float ms = 0.f;
-  if (e == hipSuccess && es == hipSuccess) hipEventElapsedTime(&ms, e0, e1);
-  hipEventDestroy(e0);
-  hipEventDestroy(e1);
-  if (e != hipSuccess) return hip_fail(e, "attn_fwd");
-  if (es != hipSuccess) return hip_fail(es, "hipEventSynchronize");
-  *ms_out = ms / iters;
   g_err[0] = 0;
   return PKH3_OK;
 }

@@ -619,6 +619,7 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
   // branch between S^T and the softmax, which lets the numerators of the first 32 keys be scheduled under
   // the MFMAs of the second 32.
   const int n_masked = (tail && t_end > t_begin && entry(t_end - 1) == nkt - 1) ? 1 : 0;
+  float ks_next = (FP8 && !HALFMODE && t_end > t_begin) ? uniform_load(kscale, entry(t_begin)) : 1.0f;
 #define PKH3_TILE_LOOP(STATIC, MASKED, FROM, TO)                                                        \
   for (int i = FROM; i < TO; ++i) {                                                                     \
     /* tile i (and, with a ring of three, i+1) is in LDS for every wave (own slices: vmcnt, the others': */ \
@@ -626,8 +627,10 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
     __syncthreads();                                                                                    \
     const char* kbuf = lds[slot];                                                                       \
-    const int tile = entry(i);                                                                          \
-    const float ks = FP8 ? uniform_load(kscale, tile) : 1.0f;                                           \
+    /* the K scale of this tile was asked for an iteration ago (with power-of-two scales the first MFMA */ \
+    /* needs it); the one of the next tile is asked for now */                                          \
+    const float ks = ks_next;                                                                           \
+    if (FP8) ks_next = uniform_load(kscale, entry(min(i + 1, t_end - 1)));                              \
     qk_tile<FP8, LEAN, (MASKED) ? 2 : 4, POW2>(w, kbuf, kbuf + kKBytes, lane, e8m0_of(ks));             \
     /* the copies of the tile two ahead are issued under the MFMAs of S^T, not in front of them: right */ \
     /* after the barrier their scalar address chain would run in every wave at once with the pipe idle */ \
@@ -714,6 +717,9 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
     for (int a = 0; a < kStages2 - 1; ++a)
       if (a < 2 * n_mine) dma_half(a, a);
     int st2 = 0, st2_free = kStages2 - 1;  // stage of half tile `it`, and the one the newest copy goes to
+    // list entry and K scale of the half tile an iteration uses are asked for an iteration ahead
+    int tile_next = n_mine > 0 ? uniform_load(mine, 0) : 0;
+    float ks2_next = (FP8 && n_mine > 0) ? uniform_load(kscale, tile_next) : 1.0f;
 #define PKH3_HALF_LOOP(STATIC)                                                                          \
   for (int it = 0; it < n_iter; ++it) {                                                                 \
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                    \
@@ -723,9 +729,11 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
     st2_free = st2;                                                                                     \
     st2 = st2 == kStages2 - 1 ? 0 : st2 + 1;                                                            \
     if (it >= 2 * n_mine) continue; /* wave-uniform: this row-block has run out of tiles (and of copies) */ \
-    const int tile = uniform_load(mine, it >> 1);                                                       \
+    const int tile = tile_next;                                                                         \
+    const float ks = ks2_next;                                                                          \
+    tile_next = uniform_load(mine, min(it + 1, 2 * n_mine - 1) >> 1);                                   \
+    if (FP8) ks2_next = uniform_load(kscale, tile_next);                                                \
     /* the running-max copy needs registers for the rescale: it takes the lean read-ahead (4 images) */ \
-    const float ks = FP8 ? uniform_load(kscale, tile) : 1.0f;                                           \
     qk_half<FP8, !STATIC, POW2>(w, hbuf, hbuf + kKHalf, lane, e8m0_of(ks));                             \
     /* copies of the next half tile of this row-block: under the MFMAs of S^T (see the whole-tile loop) */ \
     if (it + kStages2 - 1 < 2 * n_mine) dma_half(it + kStages2 - 1, st2_write);                         \

@@ -297,8 +297,8 @@ def attention_prepared(q: torch.Tensor, kv: PreparedKV, *, out: Optional[torch.T
 
 def time_attention_kernel(q, k, v, *, iters: int = 10, **opts) -> float:
     """Mean milliseconds per launch of the attention kernel alone (prologue excluded), measured with
-    HIP events inside the library on the current stream."""
-    lib = _lib.load()
+    HIP events on the current stream inside the measurement library (``libpkh3attn_bench.so``)."""
+    lib = _lib.load_bench()
     out = torch.empty_like(q)
     args, keep = fill_args(q, k, v, out, **opts)
     ws = torch.empty(workspace_bytes(args), dtype=torch.uint8, device=q.device)

@@ -16,9 +16,14 @@ def test_header_symbols_are_exported(lib):
     inc = os.path.join(ROOT, "include")
     header = "".join(open(os.path.join(inc, f)).read() for f in sorted(os.listdir(inc)) if f.endswith(".h"))
     declared = set(re.findall(r"\b(pkh3_[a-z0-9_]+)\s*\(", header))
-    assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
-    for name in declared:
+    assert declared == set(_lib.EXPORTS) | set(_lib.BENCH_EXPORTS), declared ^ (set(_lib.EXPORTS) | set(_lib.BENCH_EXPORTS))
+    for name in _lib.EXPORTS:
         assert getattr(lib, name) is not None
+    # the call that synchronises lives in the measurement library, not in the product library
+    bench = _lib.load_bench()
+    for name in _lib.BENCH_EXPORTS:
+        assert getattr(bench, name) is not None
+        assert not hasattr(lib, name)
 
 
 def test_version_and_strerror(lib):
@@ -122,7 +127,8 @@ def test_rope_tables_argument_errors(lib):
     assert lib.pkh3_rope_tables(0x1000, 4, odd, 1e4, 0x1000, 0x2000, None) == _lib.PKH3_EARG
 
 
-def test_time_kernel_argument_errors(lib):
+def test_time_kernel_argument_errors():
+    lib = _lib.load_bench()
     a = _valid_args()
     assert lib.pkh3_attn_time_kernel(C.byref(a), None, 1, None) == _lib.PKH3_ENULL
     ms = C.c_float()
