@@ -259,7 +259,7 @@ def prepare_kv(k: torch.Tensor, v: torch.Tensor, *, q_rows: Optional[int] = None
     if block_sparse:
         # size with a block map present (only the pointers' presence matters to the sizing call)
         args.blk_row_ptr = args.blk_col_idx = k.data_ptr()
-        need = workspace_bytes(args)
+        need = max(need, workspace_bytes(args))   # dense calls carry scratch of their own kind: room for either
         args.blk_row_ptr = args.blk_col_idx = None
     ws = torch.empty(need, dtype=torch.uint8, device=k.device)
     args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()

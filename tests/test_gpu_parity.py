@@ -394,3 +394,25 @@ def test_prepared_keys_serve_several_calls(variant):
         pk.attention_prepared(q, kv, k_norm_weight=wk, **q_opts)
     with pytest.raises(ValueError, match="heads"):
         pk.attention_prepared(_rand((B, Sq, H + 1, D), gen).to(dev), kv, **q_opts)
+
+
+def test_prepared_keys_workspace_holds_dense_and_block_sparse_calls():
+    """Keys prepared with ``block_sparse=True`` at a size where long dense calls bring scratch of their own (the partial
+    results of a shared last round): the workspace must hold either kind of call, and both must give the bits of the
+    direct calls."""
+    import pika_h3_flex_amd as pk
+
+    B, S, H, D = 1, 1500, 24, 128
+    gen = torch.Generator().manual_seed(17)
+    dev = "cuda"
+    q, k, v = (_rand((B, S, H, D), gen).to(dev) for _ in range(3))
+    w = torch.ones(D, device=dev)
+    kv = pk.prepare_kv(k, v, q_rows=S, block_sparse=True, k_norm_weight=w)
+    nt = (S + 63) // 64
+    tm = (torch.rand((nt, nt), generator=gen) < 0.4) | torch.eye(nt, dtype=torch.bool)
+    bm = pk.BlockMask.from_dense(tm, device=dev)
+    dense = pk.attention_prepared(q, kv, q_norm_weight=w)
+    sparse = pk.attention_prepared(q, kv, q_norm_weight=w, block_mask=bm)
+    torch.cuda.synchronize()
+    assert torch.equal(dense, pk.attention(q, k, v, q_norm_weight=w, k_norm_weight=w))
+    assert torch.equal(sparse, pk.attention(q, k, v, q_norm_weight=w, k_norm_weight=w, block_mask=bm))
