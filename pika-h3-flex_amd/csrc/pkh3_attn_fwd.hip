@@ -24,7 +24,7 @@
 // scalar: no cross-lane traffic in the rescale, none between the two GEMMs.  O leaves through LDS, turned
 // around into whole 256-byte rows.
 //
-// Other forms of the dense kernel (see attn_fwd_kernel): the short-key form (at most 16 key tiles: 4 waves per
+// Other forms of the dense kernel (see attn_fwd_body): the short-key form (at most 16 key tiles: 4 waves per
 // workgroup, 32-key half tiles, three workgroups per CU), and the long form with the key tiles of a unit shared out
 // among several workgroups that merge through global scratch, for a thinly filled last round of a long call.
 //
@@ -306,7 +306,7 @@ __device__ __forceinline__ void softmax_pv_tile(WaveState<FP8>& w, const char* v
   }
 }
 
-// ---- 32-key half tiles: the short-key and split forms of the dense kernel, phase 2 of the block-sparse one ----
+// ---- 32-key half tiles: the short-key form of the dense kernel, phase 2 of the block-sparse one ----
 // S^T (32 keys x 32 queries) into w.s[0..1]; kbuf/vbuf point at this half's K images (8 bf16 / 4 fp8 chunks)
 // and V images (8).
 // LEAN (three waves per SIMD): the K reads run 4 images ahead and only the fp8 path prefetches V (4 images).
