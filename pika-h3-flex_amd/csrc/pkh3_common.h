@@ -86,8 +86,34 @@ __device__ __forceinline__ void load_row(float (&x)[64], const __bf16* row, bool
     for (int j = 0; j < 8; ++j) x[ks * 8 + j] = valid ? (float)t[ks][j] : 0.f;
 }
 
-__device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform& t, int64_t table_row, bool valid,
-                                              int hh) {
+// The rotation tables of one row as this lane uses them (16 vectors of 4): loaded once per row, they serve every
+// head of that row.  Interleaved pairs (2i, 2i+1): c[ks] holds the pairs 8*ks + 4*hh .. +3 of this lane's elements
+// 2jj, 2jj+1.  Half-split pairs (i, i + 64): element d < 64 of this lane sits at ks < 4, its partner at ks + 4, and
+// c[2*ks], c[2*ks + 1] hold the pairs 16*ks + 8*hh .. +7.
+struct RopeRow {
+  f32x4 c[8], s[8];
+};
+
+__device__ __forceinline__ void load_rope_row(RopeRow& r, const RowTransform& t, int64_t table_row, int hh) {
+  const float* ct = t.cos_t + table_row * (kD / 2);
+  const float* st = t.sin_t + table_row * (kD / 2);
+  if (t.rope_mode == 1) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      r.c[ks] = *(const f32x4*)(ct + 8 * ks + 4 * hh);
+      r.s[ks] = *(const f32x4*)(st + 8 * ks + 4 * hh);
+    }
+  } else if (t.rope_mode == 2) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      r.c[2 * ks] = *(const f32x4*)(ct + 16 * ks + 8 * hh), r.c[2 * ks + 1] = *(const f32x4*)(ct + 16 * ks + 8 * hh + 4);
+      r.s[2 * ks] = *(const f32x4*)(st + 16 * ks + 8 * hh), r.s[2 * ks + 1] = *(const f32x4*)(st + 16 * ks + 8 * hh + 4);
+    }
+  }
+}
+
+// RMSNorm and rotation of this lane's 64 elements of a row, with the row's tables already in registers
+__device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform& t, const RopeRow& r, bool valid, int hh) {
   if (t.norm_w) {
     float ssq = 0.f;
 #pragma unroll
@@ -108,37 +134,34 @@ __device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform
     }
   }
   if (t.rope_mode == 1 && valid) {
-    // interleaved pairs (2i, 2i+1): pair index 8*ks + 4*hh + jj for this lane's elements 2jj, 2jj+1
-    const float* ct = t.cos_t + table_row * (kD / 2);
-    const float* st = t.sin_t + table_row * (kD / 2);
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      const f32x4 c = *(const f32x4*)(ct + 8 * ks + 4 * hh);
-      const f32x4 s = *(const f32x4*)(st + 8 * ks + 4 * hh);
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
         const float a0 = x[ks * 8 + 2 * jj], a1 = x[ks * 8 + 2 * jj + 1];
-        x[ks * 8 + 2 * jj] = a0 * c[jj] - a1 * s[jj];
-        x[ks * 8 + 2 * jj + 1] = a1 * c[jj] + a0 * s[jj];
+        x[ks * 8 + 2 * jj] = a0 * r.c[ks][jj] - a1 * r.s[ks][jj];
+        x[ks * 8 + 2 * jj + 1] = a1 * r.c[ks][jj] + a0 * r.s[ks][jj];
       }
     }
   } else if (t.rope_mode == 2 && valid) {
-    // half-split pairs (i, i + 64): element d < 64 of this lane sits at ks < 4, its partner at ks + 4
-    const float* ct = t.cos_t + table_row * (kD / 2);
-    const float* st = t.sin_t + table_row * (kD / 2);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      const f32x4 c0 = *(const f32x4*)(ct + 16 * ks + 8 * hh), c1 = *(const f32x4*)(ct + 16 * ks + 8 * hh + 4);
-      const f32x4 s0 = *(const f32x4*)(st + 16 * ks + 8 * hh), s1 = *(const f32x4*)(st + 16 * ks + 8 * hh + 4);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float cj = j < 4 ? c0[j & 3] : c1[j & 3], sj = j < 4 ? s0[j & 3] : s1[j & 3];
+        const float cj = j < 4 ? r.c[2 * ks][j & 3] : r.c[2 * ks + 1][j & 3], sj = j < 4 ? r.s[2 * ks][j & 3] : r.s[2 * ks + 1][j & 3];
         const float lo = x[ks * 8 + j], hi = x[(ks + 4) * 8 + j];
         x[ks * 8 + j] = lo * cj - hi * sj;
         x[(ks + 4) * 8 + j] = hi * cj + lo * sj;
       }
     }
   }
+}
+
+__device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform& t, int64_t table_row, bool valid,
+                                              int hh) {
+  RopeRow r;
+  if (t.rope_mode != 0 && valid) load_rope_row(r, t, table_row, hh);
+  norm_rope_row(x, t, r, valid, hh);
 }
 
 __device__ __forceinline__ float wave_sum_groups(float x) {

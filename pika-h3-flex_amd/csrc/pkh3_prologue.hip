@@ -57,83 +57,98 @@ hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int
 // two 32-row halves `sub`, the 64 elements d = 16*ks + 8*hh + j of row 32*sub + r -- whole 16-byte
 // pieces of the operand images, so norm and rotation need one cross-lane exchange only (the sum of
 // squares with lane l^32) and the store is 16 bytes per piece at its place in the image.
+// A wave walks kPrologueHeads consecutive heads of its rows with the rows' rotation tables in registers: the tables
+// are as many bytes per row as a head of the row itself, and every head needs them.
+constexpr int kPrologueHeads = 4;
+
 template <bool FP8>
 __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  // heads vary fastest across workgroups: neighbouring workgroups then read neighbouring 256-byte pieces of
+  // head groups vary fastest across workgroups: neighbouring workgroups then read neighbouring pieces of
   // the same [S, H, D] rows at the same time
   const int blk = blockIdx.y * 4 + wave;
   if (blk >= p.nBlk64) return;
-  const int h = blockIdx.x, b = blockIdx.z;
+  const int h0 = blockIdx.x * kPrologueHeads, b = blockIdx.z;
   const int r = lane & 31, hh = lane >> 5;
   const int rows = p.row_cnt ? p.row_cnt[b] : p.S;
-  const __bf16* xb = (const __bf16*)p.x + (int64_t)b * p.sb + (int64_t)h * p.sh;
-
   const RowTransform tf{p.norm_w, p.eps, p.rope_mode, p.cos_t, p.sin_t};
-  float x[2][64];
+
+  RopeRow rope[2];
+  int src[2];
+  bool valid[2];
 #pragma unroll
   for (int sub = 0; sub < 2; ++sub) {
     const int row = blk * 64 + sub * 32 + r;
-    const bool valid = row < rows;
-    int src = 0;
-    if (valid) src = p.gather_idx ? p.gather_idx[(int64_t)b * p.S + row] : row;
-    load_row(x[sub], xb + (int64_t)src * p.ss, valid, hh);
-    norm_rope_row(x[sub], tf, src, valid, hh);
+    valid[sub] = row < rows;
+    src[sub] = 0;
+    if (valid[sub]) src[sub] = p.gather_idx ? p.gather_idx[(int64_t)b * p.S + row] : row;
+    if (p.rope_mode != 0 && valid[sub]) load_rope_row(rope[sub], tf, src[sub], hh);
   }
 
-  if (p.norm_max) {
-    // largest row norm of this (batch, head) after norm and rotation: an upper bound for every logit is
-    // |q_i| * max_j |k_j|, which lets the attention kernel drop the running max when the bound is small
-    float nmax = 0.f;
+#pragma unroll 1
+  for (int h = h0; h < min(h0 + kPrologueHeads, p.H); ++h) {
+    const __bf16* xb = (const __bf16*)p.x + (int64_t)b * p.sb + (int64_t)h * p.sh;
+    float x[2][64];
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
-      float ssq = 0.f;
-#pragma unroll
-      for (int i = 0; i < 64; ++i) ssq += x[sub][i] * x[sub][i];
-      ssq += xhalf(ssq);
-      nmax = fmaxf(nmax, ssq);
+      load_row(x[sub], xb + (int64_t)src[sub] * p.ss, valid[sub], hh);
+      norm_rope_row(x[sub], tf, rope[sub], valid[sub], hh);
     }
-    nmax = sqrtf(wave_max(nmax));
-    if (lane == 0) atomicMax(p.norm_max + b * p.H + h, __float_as_uint(nmax));  // non-negative floats order like uints
-  }
-  char* ob = p.out + (int64_t)(b * p.H + h) * p.out_bh_stride + (int64_t)blk * p.out_blk_stride;
-  if constexpr (!FP8) {
+
+    if (p.norm_max) {
+      // largest row norm of this (batch, head) after norm and rotation: an upper bound for every logit is
+      // |q_i| * max_j |k_j|, which lets the attention kernel drop the running max when the bound is small
+      float nmax = 0.f;
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub)
+      for (int sub = 0; sub < 2; ++sub) {
+        float ssq = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        bf16x8 t;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[sub][ks * 8 + j];
-        *(bf16x8*)(ob + k_piece_offset(32 * sub + r, 2 * ks + hh)) = t;
+        for (int i = 0; i < 64; ++i) ssq += x[sub][i] * x[sub][i];
+        ssq += xhalf(ssq);
+        nmax = fmaxf(nmax, ssq);
       }
-  } else {
-    float amax = 0.f;
+      nmax = sqrtf(wave_max(nmax));
+      if (lane == 0) atomicMax(p.norm_max + b * p.H + h, __float_as_uint(nmax));  // non-negative floats order like uints
+    }
+    char* ob = p.out + (int64_t)(b * p.H + h) * p.out_bh_stride + (int64_t)blk * p.out_blk_stride;
+    if constexpr (!FP8) {
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub)
+      for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-      for (int i = 0; i < 64; ++i) amax = fmaxf(amax, fabsf(x[sub][i]));
-    amax = wave_max(amax);
-    const float scale = fp8_block_scale(amax, p.fp8_pow2 != 0);
-    const float inv = 1.0f / scale;
-    if (lane == 0) p.scale_out[(int64_t)(b * p.H + h) * p.nBlk64 + blk] = scale;
+        for (int ks = 0; ks < 8; ++ks) {
+          bf16x8 t;
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-      for (int c2 = 0; c2 < 2; ++c2) {
-        // this lane's pieces ks8 = 4*c2 .. 4*c2+3; pieces ks8 and ks8 + 2 share a lane group and a chunk
-        const i32x4 q0 = quant_fp8_chunk(x[sub], 2 * c2, inv), q1 = quant_fp8_chunk(x[sub], 2 * c2 + 1, inv);
-#pragma unroll
-        for (int a = 0; a < 2; ++a) {
-          const i32x4 t = {q0[2 * a], q0[2 * a + 1], q1[2 * a], q1[2 * a + 1]};
-          *(i32x4*)(ob + k8_chunk_offset(32 * sub + r, 2 * (4 * c2 + a) + hh)) = t;
+          for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[sub][ks * 8 + j];
+          *(bf16x8*)(ob + k_piece_offset(32 * sub + r, 2 * ks + hh)) = t;
         }
-      }
+    } else {
+      float amax = 0.f;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int i = 0; i < 64; ++i) amax = fmaxf(amax, fabsf(x[sub][i]));
+      amax = wave_max(amax);
+      const float scale = fp8_block_scale(amax, p.fp8_pow2 != 0);
+      const float inv = 1.0f / scale;
+      if (lane == 0) p.scale_out[(int64_t)(b * p.H + h) * p.nBlk64 + blk] = scale;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2) {
+          // this lane's pieces ks8 = 4*c2 .. 4*c2+3; pieces ks8 and ks8 + 2 share a lane group and a chunk
+          const i32x4 q0 = quant_fp8_chunk(x[sub], 2 * c2, inv), q1 = quant_fp8_chunk(x[sub], 2 * c2 + 1, inv);
+#pragma unroll
+          for (int a = 0; a < 2; ++a) {
+            const i32x4 t = {q0[2 * a], q0[2 * a + 1], q1[2 * a], q1[2 * a + 1]};
+            *(i32x4*)(ob + k8_chunk_offset(32 * sub + r, 2 * (4 * c2 + a) + hh)) = t;
+          }
+        }
+    }
   }
 }
 
 hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st) {
-  dim3 grid(p.H, (p.nBlk64 + 3) / 4, p.B);
+  dim3 grid((p.H + kPrologueHeads - 1) / kPrologueHeads, (p.nBlk64 + 3) / 4, p.B);
   if (p.fp8)
     hipLaunchKernelGGL(qk_prologue_kernel<true>, grid, dim3(256), 0, st, p);
   else
