@@ -72,3 +72,70 @@ def test_random_combinations(seed):
             assert cos >= 0.995 or (all_zero and err == 0.0), label
         else:
             assert err <= 2e-2 and (cos >= 0.9999 or all_zero), label
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_long_dense_calls_with_a_shared_last_round(seed):
+    """Seeded long dense calls whose query tiles overflow whole rounds of workgroups by a random amount, so that the last
+    tiles are shared out among 2 to 8 workgroups each (one or two sections, whatever the planner picks for the remainder):
+    batches, key masks (compacted key counts differ per batch), rotation, fp8 with both scale rules, large logits
+    (running-max merge).  Checked against the plain long form on the same inputs (one workgroup per query tile), for
+    identical bits on a repeated call, and against the oracle on sampled rows of the last tiles."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as O
+
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    rng = random.Random(100 + seed)
+    for case in range(10):
+        B, H = rng.choice([(1, 24), (1, 16), (2, 12), (3, 8), (1, 40)])
+        tiles = (cus + rng.randint(1, cus - 1) + B * H - 1) // (B * H)          # query tiles per (batch, head)
+        Sq = tiles * 384 - rng.randint(0, 383)
+        Sk = rng.choice([1100, 1536, 2500, 3100, 4700, 6000])
+        mode = rng.choice(["plain", "plain", "mask", "fp8", "pow2", "large"])
+        rope = rng.choice([0, 1, 2])
+        g = torch.Generator().manual_seed(5000 * seed + case)
+        q = torch.randn((B, Sq, H, D), generator=g).to(torch.bfloat16)
+        k = torch.randn((B, Sk, H, D), generator=g).to(torch.bfloat16)
+        v = torch.randn((B, Sk, H, D), generator=g).to(torch.bfloat16)
+        qw = (1.0 + 0.1 * torch.randn(D, generator=g)) * (3.5 if mode == "large" else 1.0)
+        kw = 1.0 + 0.1 * torch.randn(D, generator=g)
+        opts = dict(q_norm_weight=qw.cuda(), k_norm_weight=kw.cuda())
+        ref = dict(q_norm_weight=qw, k_norm_weight=kw)
+        if rope:
+            tq = O.rope_tables(torch.rand((Sq, 3), generator=g, dtype=torch.float64) * 30)
+            tk = O.rope_tables(torch.rand((Sk, 3), generator=g, dtype=torch.float64) * 30)
+            dev = lambda t: tuple(x.float().contiguous().cuda() for x in t)
+            opts.update(rope_mode=rope, rope_q=dev(tq), rope_k=dev(tk))
+            ref.update(rope_mode=rope, rope_q=tq, rope_k=tk)
+        if mode == "mask":
+            m = torch.rand((B, Sk), generator=g) < 0.7
+            m[B - 1, : Sk // 2] = False            # the batches keep different numbers of keys
+            opts.update(key_mask=m.cuda())
+            ref.update(key_mask=m)
+        if mode in ("fp8", "pow2"):
+            opts.update(fp8_qk=True if mode == "fp8" else "pow2")
+            ref.update(fp8_qk=True if mode == "fp8" else "pow2")
+        if mode == "large":
+            ref.update(bf16_operands=True)
+        qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+        out = pk.attention(qc, kc, vc, **opts)
+        again = pk.attention(qc, kc, vc, **opts)
+        plain = pk.attention(qc, kc, vc, long_key_kernel=True, **opts)
+        torch.cuda.synchronize()
+        label = f"seed {seed} case {case}: B={B} H={H} Sq={Sq} ({B * H * tiles} query tiles on {cus} CUs) Sk={Sk} {mode} rope={rope}"
+        assert torch.isfinite(out.float()).all(), label
+        assert torch.equal(out, again), label
+        err, cos = O.max_abs_and_cosine(out.cpu(), plain.cpu())
+        # the two forms add the same products in a different order: a bf16 step of the output at most
+        assert err <= 2.0 ** -6 * max(1.0, float(plain.float().abs().max())) and cos >= 0.99999, (label, err, cos)
+        # oracle on rows of the last query tile of the last (batch, head): tiles the shared round holds
+        rows = torch.tensor(sorted({Sq - 1, Sq - 2, Sq - 33, max(0, Sq - 200), max(0, Sq - 384), (tiles - 1) * 384}))
+        expect = O.reference_layer(q[B - 1:, :, H - 1:], k[B - 1:, :, H - 1:], v[B - 1:, :, H - 1:], q_rows=rows,
+                                   **{n: (t[B - 1:] if n == "key_mask" else t) for n, t in ref.items()})
+        got = out[B - 1:, rows.cuda()][:, :, H - 1:].cpu()
+        err, cos = O.max_abs_and_cosine(got, expect)
+        print(f"{label}: vs oracle max_abs={err:.3e} cos={cos:.6f}", flush=True)
+        if mode in ("fp8", "pow2"):
+            assert cos >= 0.995, label
+        else:
+            assert err <= 2e-2 and cos >= 0.9999, label
