@@ -121,7 +121,8 @@ WsPlan plan(const pkh3_attn_args* a, bool part_scratch = true) {
                           : (tiles384 * 8 < (size_t)kMaxPartWorkgroups ? tiles384 * 8 : (size_t)kMaxPartWorkgroups);
   w.split_bytes = part_wgs * 12 * (size_t)kPartialBytes;
   w.split_off = off;  off = align_up(off + w.split_bytes, 256);
-  w.split_cnt_off = off; off = align_up(off + part_wgs * 12 * sizeof(int), 256);
+  // positions of the work queues of a long dense call, then the arrival counters
+  w.split_cnt_off = off; off = align_up(off + (kQueueSlots + part_wgs * 12) * sizeof(int), 256);
   w.total = off;
   return w;
 }
@@ -186,7 +187,8 @@ void build(const pkh3_attn_args* a, void* workspace, Launch& L, bool part_scratc
   f.kmax = (const float*)(ws + L.w.kmax_off);
   f.split_scratch = L.w.split_bytes ? (float*)(ws + L.w.split_off) : nullptr;
   f.split_scratch_bytes = L.w.split_bytes;
-  f.split_cnt = L.w.split_bytes ? (int*)(ws + L.w.split_cnt_off) : nullptr;
+  f.split_cnt = (int*)(ws + L.w.split_cnt_off) + kQueueSlots;
+  f.queue_next = (int*)(ws + L.w.split_cnt_off);
 }
 
 int hip_fail(hipError_t e, const char* what) {

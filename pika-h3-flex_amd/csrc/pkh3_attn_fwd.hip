@@ -416,7 +416,7 @@ constexpr int fwd_lds_bytes() {
 // partial results start at slot `part_base` of the scratch, their counters at unit slot `cnt_base`).
 template <bool FP8, bool SPARSE, int WAVES, bool POW2>
 __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int unit0, int units, int parts, int part_base,
-                                              int cnt_base, char* lds_raw) {
+                                              int cnt_base, char* lds_raw, int fetched = -1) {
   static_assert(!SPARSE || WAVES == kSparseWaves, "block-sparse layout: a wave pair per row-block of the plan");
   static_assert(FP8 || !POW2, "power-of-two scales belong to the fp8 form");
   constexpr bool SHORT = !SPARSE && WAVES == kShortWaves;
@@ -440,9 +440,10 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD one contiguous run of
   // (batch, head, query tile) so the 32 CUs behind one L2 stream the same K/V at the same time.
   // (Every section of a launch starts at a workgroup index that is a multiple of 8.)
+  // (`fetched` >= 0: the unit came from the work queues instead, see attn_fwd_dense_kernel.)
   const int total = units * parts;
   const int per_xcd = (total + 7) / 8;
-  const int lin = (blk & 7) * per_xcd + (blk >> 3);
+  const int lin = fetched >= 0 ? fetched : (blk & 7) * per_xcd + (blk >> 3);
   if (lin >= total) return;
   // unit inside the section, and which share of its keys: share-major, so that the workgroups an XCD runs at the
   // same time walk the same key tiles of (mostly) the same head, as the whole units before them do
@@ -861,20 +862,60 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
   }
 }
 
-// The block-sparse kernel and the short-key dense kernel.
+// Work queues of a launch's units.  The XCDs of one part hold different clocks under the power cap
+// (a few per cent apart), and the hardware deals workgroups to them round-robin, an eighth each whatever their speed,
+// so with a fixed workgroup -> unit map the call lasts as long as its slowest XCD needs for its eighth.  Instead every
+// XCD has a queue (a counter) over its contiguous run of units: a workgroup takes the next unit of its own XCD's queue
+// and, when that is empty, of the queue with the most units left; the launch holds an eighth more workgroups than
+// units, so an XCD that is through early keeps getting workgroups, which take units off the slower ones.  A workgroup
+// that finds every queue empty exits.  Returns the unit (index inside the section) or -1.
+__device__ __forceinline__ int fetch_unit(int* queue_next, int home, int units) {
+  const int per = (units + kQueues - 1) / kQueues;
+  int q = home;
+  // Every pass either takes a unit, or finds all queues empty, or lost a unit to another workgroup (which is
+  // progress of the launch as a whole: the positions only grow), so the loop ends.
+#pragma unroll 1
+  for (;;) {
+    const int size = max(0, min(per, units - q * per));
+    // a look first: a queue that is empty stays empty, no need to count it further up
+    if (__hip_atomic_load(queue_next + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < size) {
+      const int i = __hip_atomic_fetch_add(queue_next + q, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (i < size) return q * per + i;
+    }
+    int best = -1, most = 0;
+    for (int j = 0; j < kQueues; ++j) {
+      const int left = max(0, min(per, units - j * per)) - __hip_atomic_load(queue_next + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (left > most) most = left, best = j;
+    }
+    if (best < 0) return -1;
+    q = best;
+  }
+}
+
+// The block-sparse kernel and the short-key dense kernel (the block-sparse one takes its units from the work queues
+// when the launch has them: its workgroups differ in length with the tile lists on top of the XCDs' clocks).
 template <bool FP8, bool SPARSE, int WAVES, bool POW2>
 __global__ __launch_bounds__(64 * WAVES, (SPARSE ? 8 / WAVES : 3)) void attn_fwd_kernel(FwdParams p) {
   __shared__ __attribute__((aligned(1024))) char lds_raw[fwd_lds_bytes<FP8, SPARSE, WAVES>()];
-  attn_fwd_body<FP8, SPARSE, WAVES, POW2>(p, blockIdx.x, 0, p.sec_units[0], 1, 0, 0, lds_raw);
+  __shared__ int fetched_unit;
+  int fetched = -1;
+  if (p.queue_next) {   // wave-uniform
+    if (threadIdx.x == 0) fetched_unit = fetch_unit(p.queue_next, blockIdx.x & (kQueues - 1), p.sec_units[0]);
+    __syncthreads();
+    fetched = __builtin_amdgcn_readfirstlane(fetched_unit);
+    if (fetched < 0) return;
+  }
+  attn_fwd_body<FP8, SPARSE, WAVES, POW2>(p, blockIdx.x, 0, p.sec_units[0], 1, 0, 0, lds_raw, fetched);
 }
 
 // The long dense kernel: a launch of up to kSections sections, handed out in this order as CUs fall free.  Section 0
 // holds whole units (one workgroup each); the later ones the units of a thinly filled last round, each shared out
-// among sec_parts[] workgroups.
+// among sec_parts[] workgroups.  When the launch has work queues, every section's work is taken from queues of its own.
 template <bool FP8, bool POW2>
 __global__ __launch_bounds__(64 * kDenseWaves, 1) void attn_fwd_dense_kernel(FwdParams p) {
   __shared__ __attribute__((aligned(1024))) char lds_raw[fwd_lds_bytes<FP8, false, kDenseWaves>()];
-  static_assert(kSections == 3, "the section look-up below is written out for three");
+  __shared__ int fetched_unit;
+  static_assert(kSections == 3 && kSections * kQueues <= kQueueSlots, "the section look-up below is written out for three");
   const int bid = blockIdx.x, b0 = p.sec_blocks[0], b1 = p.sec_blocks[1];
   const int sec = (bid >= b0 ? 1 : 0) + (bid >= b0 + b1 ? 1 : 0);
   const int blk = bid - (sec >= 1 ? b0 : 0) - (sec >= 2 ? b1 : 0);
@@ -884,7 +925,14 @@ __global__ __launch_bounds__(64 * kDenseWaves, 1) void attn_fwd_dense_kernel(Fwd
   // partial results and counters of section 2 lie behind those of section 1 (section 0 has none)
   const bool behind = sec == 2 && p.sec_parts[1] > 1;
   const int part_base = behind ? p.sec_units[1] * p.sec_parts[1] : 0, cnt_base = behind ? p.sec_units[1] : 0;
-  attn_fwd_body<FP8, false, kDenseWaves, POW2>(p, blk, unit0, units, parts, part_base, cnt_base, lds_raw);
+  int fetched = -1;
+  if (p.queue_next) {   // wave-uniform; every section has queues of its own over its workgroups' work
+    if (threadIdx.x == 0) fetched_unit = fetch_unit(p.queue_next + sec * kQueues, blk & (kQueues - 1), units * parts);
+    __syncthreads();
+    fetched = __builtin_amdgcn_readfirstlane(fetched_unit);
+    if (fetched < 0) return;
+  }
+  attn_fwd_body<FP8, false, kDenseWaves, POW2>(p, blk, unit0, units, parts, part_base, cnt_base, lds_raw, fetched);
 }
 
 static int blocks_of(int workgroups) { return (workgroups + 7) / 8 * 8; }
@@ -925,11 +973,22 @@ static hipError_t launch_fp(FwdParams p, int cus, hipStream_t st) {
   auto units = [&](int blocks) { return p.B * p.H * ((nQ32 + blocks - 1) / blocks); };
   for (int i = 0; i < kSections; ++i) p.sec_units[i] = p.sec_blocks[i] = 0, p.sec_parts[i] = 1;
   if (p.plan) {
-    p.sec_units[0] = units(kSparseWaves);
-    hipLaunchKernelGGL((attn_fwd_kernel<FP8, true, kSparseWaves, POW2>), dim3(blocks_of(p.sec_units[0])), dim3(64 * kSparseWaves), 0, st, p);
+    const int n = units(kSparseWaves);
+    p.sec_units[0] = n;
+    int wgs = n;
+    if (p.queue_next && cus > 0 && n >= cus) {
+      // at least a round of workgroups: units from the work queues, an eighth more workgroups than units
+      hipError_t e = launch_fill_zero((unsigned*)p.queue_next, kQueues, st);
+      if (e != hipSuccess) return e;
+      wgs += max(kQueues, n / 8);
+    } else {
+      p.queue_next = nullptr;
+    }
+    hipLaunchKernelGGL((attn_fwd_kernel<FP8, true, kSparseWaves, POW2>), dim3(blocks_of(wgs)), dim3(64 * kSparseWaves), 0, st, p);
     return hipGetLastError();
   }
   if (p.nKt <= kShortMaxTiles && !p.long_key_kernel) {
+    p.queue_next = nullptr;
     p.sec_units[0] = units(kShortWaves);
     hipLaunchKernelGGL((attn_fwd_kernel<FP8, false, kShortWaves, POW2>), dim3(blocks_of(p.sec_units[0])), dim3(64 * kShortWaves), 0, st, p);
     return hipGetLastError();
@@ -937,21 +996,33 @@ static hipError_t launch_fp(FwdParams p, int cus, hipStream_t st) {
   const int n = units(kDenseWaves);
   const int whole = cus > 0 ? n / cus * cus : n, rest = n - whole;
   p.sec_units[0] = n;
-  if (whole > 0 && rest > 0 && !p.long_key_kernel && p.split_cnt) {
+  int shared = 0;   // units whose key tiles are shared out: they have arrival counters
+  if (whole > 0 && rest > 0 && !p.long_key_kernel && p.split_cnt && p.split_scratch_bytes) {
     const int64_t cap = (int64_t)(p.split_scratch_bytes / ((size_t)kDenseWaves * kMergeBytes));
     const TailPlan t = plan_tail(rest, cus, p.nKt, cap);
     if (t.parts[0] > 1 || t.parts[1] > 1) {
       p.sec_units[0] = whole;
       p.sec_units[1] = t.units[0], p.sec_parts[1] = t.parts[0];
       p.sec_units[2] = t.units[1], p.sec_parts[2] = t.parts[1];
-      // the arrival counters of the shared units start at zero
-      const int shared = (t.parts[0] > 1 ? t.units[0] : 0) + (t.parts[1] > 1 ? t.units[1] : 0);
-      hipError_t e = launch_fill_zero((unsigned*)p.split_cnt, shared * kDenseWaves, st);
-      if (e != hipSuccess) return e;
+      shared = (t.parts[0] > 1 ? t.units[0] : 0) + (t.parts[1] > 1 ? t.units[1] : 0);
     }
   }
+  // calls of at least one round of workgroups take their whole units from the work queues
+  const bool queues = whole > 0 && !p.long_key_kernel && p.queue_next;
+  if (!queues) p.queue_next = nullptr;
+  if (queues || shared > 0) {
+    // queue positions and arrival counters start at zero (the arrival counters follow the queue slots)
+    hipError_t e = launch_fill_zero((unsigned*)(p.split_cnt - kQueueSlots), kQueueSlots + shared * kDenseWaves, st);
+    if (e != hipSuccess) return e;
+  }
   int blocks = 0;
-  for (int i = 0; i < kSections; ++i) blocks += p.sec_blocks[i] = blocks_of(p.sec_units[i] * p.sec_parts[i]);
+  for (int i = 0; i < kSections; ++i) {
+    int wgs = p.sec_units[i] * p.sec_parts[i];
+    // the spare workgroups of the faster XCDs: an eighth on top of the whole units; as many again for the shared
+    // units of the call's end, where an XCD that is through early can take most of a slower one's share
+    if (queues && wgs > 0) wgs += i == 0 ? max(kQueues, wgs / 8) : wgs;
+    blocks += p.sec_blocks[i] = blocks_of(wgs);
+  }
   hipLaunchKernelGGL((attn_fwd_dense_kernel<FP8, POW2>), dim3(blocks), dim3(64 * kDenseWaves), 0, st, p);
   return hipGetLastError();
 }

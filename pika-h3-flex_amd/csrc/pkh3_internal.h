@@ -19,6 +19,8 @@ constexpr int kSparseLists = 1 + kSparseRows;
 constexpr int kPartialBytes = 64 * 64 * 4 + 4 * 64 * 4;
 constexpr int kMaxPartWorkgroups = 512;
 constexpr int kSections = 3;     // sections of a long dense launch
+constexpr int kQueues = 8;       // work queues of a long dense launch: one per XCD
+constexpr int kQueueSlots = 64;  // ints set aside for their positions, in front of the arrival counters
 constexpr int kShortMaxTiles = 16;  // dense calls with at most this many key tiles run the short-key kernel
 
 // Where each intermediate lives inside the caller's workspace (byte offsets, 256-aligned).
@@ -95,7 +97,8 @@ struct FwdParams {
   // wave of a unit of the call's last round)
   float* split_scratch;
   size_t split_scratch_bytes;
-  int* split_cnt;
+  int* split_cnt;           // arrival counters; the kQueueSlots ints in front of them belong to the work queues
+  int* queue_next;          // [kQueues] next unit of each work queue (= split_cnt - kQueueSlots), or null: fixed map
   // filled per launch: the sections of the launch.  A unit is one workgroup's block of queries; section i covers
   // sec_units[i] units after those of the sections before it, sec_parts[i] workgroups per unit, in sec_blocks[i]
   // workgroup indices (a multiple of 8)
