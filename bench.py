@@ -34,14 +34,14 @@ HBM_PEAK_GBS = 8000.0
 # factors from a 1 GiB copy) in earlier profiling runs of the same command, not in this run: (bytes, file that holds
 # the counter values and the commands)
 MEASURED_TRAFFIC = {
-    "480p": (4.49e9, "profiles/attn_fwd_dense_kernel_480p_bf16.md"),
-    "480p-fp8": (3.76e9, "profiles/attn_fwd_dense_kernel_480p_fp8.md"),
-    "480p-fp8-pow2": (3.76e9, "profiles/attn_fwd_dense_kernel_480p_fp8.md"),
+    "480p": (4.57e9, "profiles/attn_fwd_dense_kernel_480p_bf16.md"),
+    "480p-fp8": (3.84e9, "profiles/attn_fwd_dense_kernel_480p_fp8.md"),
+    "480p-fp8-pow2": (3.81e9, "profiles/attn_fwd_dense_kernel_480p_fp8.md"),
     "480p-sparse-fp8-pow2": (2.118e10, "profiles/attn_fwd_kernel_480p_sparse_fp8.md"),
-    "480p-sparse": (3.160e10, "profiles/attn_fwd_kernel_480p_sparse_bf16.md"),
+    "480p-sparse": (3.213e10, "profiles/attn_fwd_kernel_480p_sparse_bf16.md"),
     "480p-sparse-fp8": (2.129e10, "profiles/attn_fwd_kernel_480p_sparse_fp8.md"),
-    "768p": (2.06e10, "profiles/attn_fwd_dense_kernel_768p_bf16.md"),
-    "joint": (4.49e9, "profiles/attn_fwd_dense_kernel_joint_bf16.md"),
+    "768p": (2.33e10, "profiles/attn_fwd_dense_kernel_768p_bf16.md"),
+    "joint": (4.55e9, "profiles/attn_fwd_dense_kernel_joint_bf16.md"),
     "cross": (6.15e8, "profiles/attn_fwd_kernel_cross_short_key.md"),
 }
 GEMM_TRAFFIC = (7.51e9, "profiles/gemm_kernel_480p_block.md")  # to_q/to_k/to_v launch of the 480p block
