@@ -130,7 +130,11 @@ typedef struct pkh3_attn_args {
   const int32_t* blk_row_ptr;
   const int32_t* blk_col_idx;
   uint32_t flags;
-  /* scratch, 256-byte aligned, at least pkh3_workspace_bytes() long */
+  /* scratch, 256-byte aligned, at least pkh3_workspace_bytes() long.  It must stay alive until the stream has
+     run the call.  Every call writes in it (behind the keys, also with PKH3_FLAG_KV_PREPARED: block-sparse plans,
+     work-queue positions, arrival counters and partial results of workgroups that share a query tile), so
+     calls that may overlap on one GPU -- different streams -- need a workspace each; calls on one stream are
+     ordered and may share one */
   void* workspace;
   size_t workspace_bytes;
 } pkh3_attn_args;
