@@ -139,3 +139,68 @@ def test_random_long_dense_calls_with_a_shared_last_round(seed):
             assert cos >= 0.995, label
         else:
             assert err <= 2e-2 and cos >= 0.9999, label
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_block_sparse_calls_that_fill_the_part(seed):
+    """Seeded block-sparse calls with more workgroups than the part has CUs, the size from which their units are handed
+    out through the per-XCD work queues: random tile maps (density 0.03 to 0.5) with some row-blocks that keep nothing
+    and some that keep everything, so that the workgroups' tile lists differ widely in length; rectangular lengths,
+    rotation, fp8 with both scale rules.  Checked for identical bits on a repeated call and against the oracle on
+    sampled rows of the first, last, an empty and a full row-block."""
+    import pika_h3_flex_amd as pk
+    from oracle import attention_oracle as O
+
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    rng = random.Random(300 + seed)
+    for case in range(8):
+        B, H = rng.choice([(1, 24), (1, 16), (2, 12), (3, 8)])
+        groups = (cus + rng.randint(1, 2 * cus) + B * H - 1) // (B * H)        # workgroups (4 row-blocks) per (batch, head)
+        Sq = groups * 256 - rng.randint(0, 255)
+        Sk = Sq if rng.random() < 0.5 else rng.choice([700, 1536, 2500, 4100])
+        mode = rng.choice(["bf16", "bf16", "fp8", "pow2"])
+        rope = rng.choice([0, 1, 2]) if Sq == Sk else 0
+        g = torch.Generator().manual_seed(9000 * seed + case)
+        q = torch.randn((B, Sq, H, D), generator=g).to(torch.bfloat16)
+        k = torch.randn((B, Sk, H, D), generator=g).to(torch.bfloat16)
+        v = torch.randn((B, Sk, H, D), generator=g).to(torch.bfloat16)
+        qw = 1.0 + 0.1 * torch.randn(D, generator=g)
+        kw = 1.0 + 0.1 * torch.randn(D, generator=g)
+        opts = dict(q_norm_weight=qw.cuda(), k_norm_weight=kw.cuda())
+        ref = dict(q_norm_weight=qw, k_norm_weight=kw)
+        if rope:
+            tabs = O.rope_tables(torch.rand((Sq, 3), generator=g, dtype=torch.float64) * 30)
+            opts.update(rope_mode=rope, rope_q=tuple(t.float().contiguous().cuda() for t in tabs))
+            ref.update(rope_mode=rope, rope_q=tabs)
+        nq, nk = (Sq + 63) // 64, (Sk + 63) // 64
+        tm = torch.rand((nq, nk), generator=g) < rng.choice([0.03, 0.1, 0.25, 0.5])
+        empty, full = rng.randrange(1, nq - 1), rng.randrange(1, nq - 1)
+        tm[empty] = False
+        tm[full] = True
+        opts.update(block_mask=pk.BlockMask.from_dense(tm, device="cuda"))
+        ref.update(tile_map=tm)
+        if mode != "bf16":
+            opts.update(fp8_qk=True if mode == "fp8" else "pow2")
+            ref.update(fp8_qk=True if mode == "fp8" else "pow2")
+        qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+        out = pk.attention(qc, kc, vc, **opts)
+        again = pk.attention(qc, kc, vc, **opts)
+        torch.cuda.synchronize()
+        label = (f"seed {seed} case {case}: B={B} H={H} Sq={Sq} ({B * H * groups} workgroups on {cus} CUs) Sk={Sk} {mode} "
+                 f"rope={rope} density={float(tm.float().mean()):.3f}")
+        assert torch.isfinite(out.float()).all(), label
+        assert torch.equal(out, again), label
+        if empty != full:
+            assert float(out[:, empty * 64:(empty + 1) * 64].float().abs().max()) == 0.0, label   # keeps nothing: zeros
+        rows = sorted({0, 63, Sq - 1, (nq - 1) * 64, empty * 64 + 5, full * 64, full * 64 + 37,
+                       min(Sq - 1, full * 64 + 63), rng.randrange(Sq), rng.randrange(Sq), rng.randrange(Sq)})
+        rows = torch.tensor(rows)
+        expect = torch.nan_to_num(O.reference_layer(q[B - 1:, :, H - 1:], k[B - 1:, :, H - 1:], v[B - 1:, :, H - 1:],
+                                                    q_rows=rows, **ref), nan=0.0)
+        got = out[B - 1:, rows.cuda()][:, :, H - 1:].cpu()
+        err, cos = O.max_abs_and_cosine(got, expect)
+        print(f"{label}: vs oracle max_abs={err:.3e} cos={cos:.6f}", flush=True)
+        if mode != "bf16":
+            assert cos >= 0.995, label
+        else:
+            assert err <= 2e-2 and cos >= 0.9999, label
