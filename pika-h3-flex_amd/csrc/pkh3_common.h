@@ -24,9 +24,10 @@
 //       16*kb + c -- the same lane-to-d assignment as the bf16 images; Q uses it alike, which is all the
 //       contraction needs.
 //
-// Rows are prepared (RMSNorm, rotation, quantisation) with two lanes per row: lane (r = l % 32, hh = l / 32)
-// holds the 64 elements d = 16*ks8 + 8*hh + j of row r, i.e. the 8-element pieces p8 = 2*ks8 + hh of the row.
-// Piece p8 of a row belongs to lane group g = p8 % 4 and k-step ks = p8 / 4 of the images above.
+// K rows are prepared (RMSNorm, rotation, quantisation) in the layout of the images themselves, four lanes per row
+// (norm_rope_quarter below).  The attention kernel prepares its Q rows with two lanes per row: lane (r = l % 32,
+// hh = l / 32) holds the 64 elements d = 16*ks8 + 8*hh + j of row r, i.e. the 8-element pieces p8 = 2*ks8 + hh of the
+// row; piece p8 of a row belongs to lane group g = p8 % 4 and k-step ks = p8 / 4 of the images above.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -63,7 +64,7 @@ __device__ __forceinline__ float wave_max(float x) {
   return x;
 }
 
-// RMSNorm + rotation of one row, shared by the K prologue and the attention kernel's Q load.
+// RMSNorm + rotation of one row, two lanes per row (the attention kernel's Q load).
 // `x` holds this lane's 64 elements d = 16*ks + 8*hh + j (index ks*8 + j) of the row; lane l^32 holds
 // the other 64, so the sum of squares needs one exchange and both pairings of the rotation
 // (interleaved (2i,2i+1) / half-split (i,i+64)) stay inside the lane.
@@ -86,8 +87,7 @@ __device__ __forceinline__ void load_row(float (&x)[64], const __bf16* row, bool
     for (int j = 0; j < 8; ++j) x[ks * 8 + j] = valid ? (float)t[ks][j] : 0.f;
 }
 
-// The rotation tables of one row as this lane uses them (16 vectors of 4): loaded once per row, they serve every
-// head of that row.  Interleaved pairs (2i, 2i+1): c[ks] holds the pairs 8*ks + 4*hh .. +3 of this lane's elements
+// The rotation tables of one row as this lane uses them (16 vectors of 4).  Interleaved pairs (2i, 2i+1): c[ks] holds the pairs 8*ks + 4*hh .. +3 of this lane's elements
 // 2jj, 2jj+1.  Half-split pairs (i, i + 64): element d < 64 of this lane sits at ks < 4, its partner at ks + 4, and
 // c[2*ks], c[2*ks + 1] hold the pairs 16*ks + 8*hh .. +7.
 struct RopeRow {
@@ -164,6 +164,15 @@ __device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform
   norm_rope_row(x, t, r, valid, hh);
 }
 
+// *slot = max(*slot, v) for non-negative floats kept as their bit patterns (they order like unsigned integers).
+// Thousands of waves raise the same few words: atomics on one address are served one after the other, so the word is
+// read first and the atomic only issued by a wave that would raise it (the value only grows, so a wave that sees an
+// older, smaller one merely issues an atomic it did not need).
+__device__ __forceinline__ void raise_max(unsigned* slot, float v) {
+  const unsigned bits = __float_as_uint(v);
+  if (bits > __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(slot, bits);
+}
+
 __device__ __forceinline__ float wave_sum_groups(float x) {
   // sum over the four lanes l % 16 == const (one per 16-lane group)
   x += __shfl_xor(x, 16, 64);
@@ -171,16 +180,112 @@ __device__ __forceinline__ float wave_sum_groups(float x) {
   return x;
 }
 
-// byte offset, inside a bf16 K tile, of the 16-byte piece p8 (elements 8*p8 .. 8*p8+7) of the tile's row rt
-__device__ __forceinline__ int k_piece_offset(int rt, int p8) {
-  const int half = rt >> 5, kb2 = (rt >> 4) & 1, c = rt & 15, ks = p8 >> 2, g = p8 & 3;
-  return ((((half * 4 + ks) * 2 + kb2) * 64) + 16 * g + c) * 16;
+// ---- four lanes per row: the layout of the 16x16 operand images themselves ----
+// Lane (c = l % 16, g = l / 16) holds the pieces p8 = 4*ks + g of row c of a 16-row block, i.e. elements
+// d = 32*ks + 8*g + j at x[8*ks + j]; the three other lane groups (lanes l ^ 16, l ^ 32, l ^ 48) hold the rest of the
+// row, so the sum of squares needs two exchanges and both pairings of the rotation (interleaved (2i, 2i+1) /
+// half-split (i, i+64): ks and ks + 2) stay inside the lane.  What a lane holds is exactly its 16 bytes of the four K
+// images (ks = 0..3) of its 16-row block, so rows prepared this way are stored without any lane movement.  Used by
+// the K prologue and by the K epilogue of the projection GEMM.  Same arithmetic as norm_rope_row.
+
+// The rotation tables of one row as its lane group uses them (8 vectors of 4).  Interleaved: c[ks] = pairs
+// 16*ks + 4*g .. +3 (elements 2jj, 2jj+1 of piece ks).  Half-split: c[2*ks], c[2*ks+1] = pairs 32*ks + 8*g .. +7
+// (element j of piece ks with its partner in piece ks + 2), ks = 0, 1.
+struct RopeQuarter {
+  f32x4 c[4], s[4];
+};
+
+__device__ __forceinline__ void load_rope_quarter(RopeQuarter& r, const RowTransform& t, int64_t table_row, int g) {
+  const float* ct = t.cos_t + table_row * (kD / 2);
+  const float* st = t.sin_t + table_row * (kD / 2);
+  if (t.rope_mode == 1) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      r.c[ks] = *(const f32x4*)(ct + 16 * ks + 4 * g);
+      r.s[ks] = *(const f32x4*)(st + 16 * ks + 4 * g);
+    }
+  } else if (t.rope_mode == 2) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      r.c[2 * ks] = *(const f32x4*)(ct + 32 * ks + 8 * g), r.c[2 * ks + 1] = *(const f32x4*)(ct + 32 * ks + 8 * g + 4);
+      r.s[2 * ks] = *(const f32x4*)(st + 32 * ks + 8 * g), r.s[2 * ks + 1] = *(const f32x4*)(st + 32 * ks + 8 * g + 4);
+    }
+  }
 }
 
-// byte offset, inside an fp8 K tile, of the 16-byte chunk that holds the pieces p8 and p8 + 4 (p8 % 8 < 4) of row rt
-__device__ __forceinline__ int k8_chunk_offset(int rt, int p8) {
-  const int kb = rt >> 4, c = rt & 15, c2 = p8 >> 3, g = p8 & 3;
-  return (((kb * 2 + c2) * 64) + 16 * g + c) * 16;
+// The RMSNorm weights of this lane's 32 elements: w[2*ks], w[2*ks + 1] = weights 32*ks + 8*g .. +7
+struct NormQuarter {
+  f32x4 w[8];
+};
+
+__device__ __forceinline__ void load_norm_quarter(NormQuarter& n, const RowTransform& t, int g) {
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    n.w[2 * ks] = *(const f32x4*)(t.norm_w + 32 * ks + 8 * g);
+    n.w[2 * ks + 1] = *(const f32x4*)(t.norm_w + 32 * ks + 8 * g + 4);
+  }
+}
+
+// RMSNorm and rotation of this lane's 32 elements of a row, with the weights and the row's tables already in registers
+__device__ __forceinline__ void norm_rope_quarter(float (&x)[32], const RowTransform& t, const NormQuarter& n, const RopeQuarter& r,
+                                                  bool valid, int g) {
+  if (t.norm_w) {
+    float ssq = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) ssq += x[i] * x[i];
+    ssq = wave_sum_groups(ssq);
+    // an all-zero row with eps == 0 stays all zero instead of 0 * inf
+    const float ms = ssq * (1.0f / kD) + t.eps;
+    const float rs = ms > 0.f ? rsqrtf(ms) : 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[ks * 8 + j] *= rs * n.w[2 * ks][j];
+        x[ks * 8 + 4 + j] *= rs * n.w[2 * ks + 1][j];
+      }
+  }
+  if (t.rope_mode == 1 && valid) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const float a0 = x[ks * 8 + 2 * jj], a1 = x[ks * 8 + 2 * jj + 1];
+        x[ks * 8 + 2 * jj] = a0 * r.c[ks][jj] - a1 * r.s[ks][jj];
+        x[ks * 8 + 2 * jj + 1] = a1 * r.c[ks][jj] + a0 * r.s[ks][jj];
+      }
+  } else if (t.rope_mode == 2 && valid) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float cj = r.c[2 * ks + (j >> 2)][j & 3], sj = r.s[2 * ks + (j >> 2)][j & 3];
+        const float lo = x[ks * 8 + j], hi = x[(ks + 2) * 8 + j];
+        x[ks * 8 + j] = lo * cj - hi * sj;
+        x[(ks + 2) * 8 + j] = hi * cj + lo * sj;
+      }
+  }
+}
+
+__device__ __forceinline__ void norm_rope_quarter(float (&x)[32], const RowTransform& t, int64_t table_row, bool valid, int g) {
+  NormQuarter n;
+  RopeQuarter r;
+  if (t.norm_w) load_norm_quarter(n, t, g);
+  if (t.rope_mode != 0 && valid) load_rope_quarter(r, t, table_row, g);
+  norm_rope_quarter(x, t, n, r, valid, g);
+}
+
+// eight values -> eight fp8 e4m3 bytes
+__device__ __forceinline__ i32x2 quant_fp8_piece(const float* x, float inv) {
+  i32x2 t;
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    int v = 0;
+    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * w] * inv, x[4 * w + 1] * inv, v, false);
+    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * w + 2] * inv, x[4 * w + 3] * inv, v, true);
+    t[w] = v;
+  }
+  return t;
 }
 
 // key (inside its 32-key half) that element j of lane group g carries in a V image / in the P operand

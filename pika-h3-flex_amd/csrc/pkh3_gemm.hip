@@ -44,72 +44,6 @@ __device__ __forceinline__ void gemm_dma16(const char* g, unsigned lane_off, cha
                : "memory", "m0");
 }
 
-// RMSNorm + rotation of a quarter row: lane group g of a token holds the pieces p8 = 4*ks + g, i.e. elements
-// d = 32*ks + 8*g + j at x[8*ks + j]; the three other lane groups (lanes l ^ 16, l ^ 32, l ^ 48) hold the rest of the
-// row, so the sum of squares needs two exchanges and both pairings of the rotation (interleaved (2i, 2i+1) /
-// half-split (i, i+64): ks and ks + 2) stay inside the lane.  Same arithmetic as norm_rope_row.
-__device__ __forceinline__ void norm_rope_quarter(float (&x)[32], const RowTransform& t, int64_t table_row, bool valid, int g) {
-  if (t.norm_w) {
-    float ssq = 0.f;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) ssq += x[i] * x[i];
-    ssq = wave_sum_groups(ssq);
-    const float ms = ssq * (1.0f / kD) + t.eps;
-    const float rs = ms > 0.f ? rsqrtf(ms) : 0.f;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const f32x4 w0 = *(const f32x4*)(t.norm_w + 32 * ks + 8 * g), w1 = *(const f32x4*)(t.norm_w + 32 * ks + 8 * g + 4);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        x[ks * 8 + j] *= rs * w0[j];
-        x[ks * 8 + 4 + j] *= rs * w1[j];
-      }
-    }
-  }
-  if (t.rope_mode == 1 && valid) {
-    const float* ct = t.cos_t + table_row * (kD / 2);
-    const float* st = t.sin_t + table_row * (kD / 2);
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const f32x4 c = *(const f32x4*)(ct + 16 * ks + 4 * g), s = *(const f32x4*)(st + 16 * ks + 4 * g);
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const float a0 = x[ks * 8 + 2 * jj], a1 = x[ks * 8 + 2 * jj + 1];
-        x[ks * 8 + 2 * jj] = a0 * c[jj] - a1 * s[jj];
-        x[ks * 8 + 2 * jj + 1] = a1 * c[jj] + a0 * s[jj];
-      }
-    }
-  } else if (t.rope_mode == 2 && valid) {
-    const float* ct = t.cos_t + table_row * (kD / 2);
-    const float* st = t.sin_t + table_row * (kD / 2);
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const f32x4 c0 = *(const f32x4*)(ct + 32 * ks + 8 * g), c1 = *(const f32x4*)(ct + 32 * ks + 8 * g + 4);
-      const f32x4 s0 = *(const f32x4*)(st + 32 * ks + 8 * g), s1 = *(const f32x4*)(st + 32 * ks + 8 * g + 4);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float cj = j < 4 ? c0[j & 3] : c1[j & 3], sj = j < 4 ? s0[j & 3] : s1[j & 3];
-        const float lo = x[ks * 8 + j], hi = x[(ks + 2) * 8 + j];
-        x[ks * 8 + j] = lo * cj - hi * sj;
-        x[(ks + 2) * 8 + j] = hi * cj + lo * sj;
-      }
-    }
-  }
-}
-
-// eight values -> eight fp8 e4m3 bytes
-__device__ __forceinline__ i32x2 quant_fp8_piece(const float* x, float inv) {
-  i32x2 t;
-#pragma unroll
-  for (int w = 0; w < 2; ++w) {
-    int v = 0;
-    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * w] * inv, x[4 * w + 1] * inv, v, false);
-    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[4 * w + 2] * inv, x[4 * w + 3] * inv, v, true);
-    t[w] = v;
-  }
-  return t;
-}
-
 template <int EPI>
 __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget& tg, int m_tile, int n_tile_in_target,
                                           char* lds_raw) {
@@ -358,7 +292,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
       }
       if (tg.norm_max) {
         nmax = sqrtf(wave_max(nmax));
-        if (lane == 0) atomicMax(tg.norm_max + head, __float_as_uint(nmax));
+        if (lane == 0) raise_max(tg.norm_max + head, nmax);
       }
       char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)tile * tg.out_blk_stride;
       if (!tg.fp8) {

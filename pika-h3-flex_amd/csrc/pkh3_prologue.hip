@@ -53,102 +53,85 @@ hipError_t launch_mask_compact(const uint8_t* mask, int B, int Sk, int* idx, int
 // ------------------------------------------------------------------------------------------------
 // RMSNorm + RoPE (+ fp8 quantisation) of K rows into operand images (the Q side does the same math
 // inside the attention kernel, on the rows each wave owns).
-// One wave owns one 64-row block of one (batch, head): lane (r = l%32, hh = l/32) holds, for the
-// two 32-row halves `sub`, the 64 elements d = 16*ks + 8*hh + j of row 32*sub + r -- whole 16-byte
-// pieces of the operand images, so norm and rotation need one cross-lane exchange only (the sum of
-// squares with lane l^32) and the store is 16 bytes per piece at its place in the image.
-// A wave walks kPrologueHeads consecutive heads of its rows with the rows' rotation tables in registers: the tables
-// are as many bytes per row as a head of the row itself, and every head needs them.
-constexpr int kPrologueHeads = 4;
-
+// One wave owns one 64-row tile of one (batch, head) and walks its four 16-row blocks, four lanes per row: lane
+// (c = l%16, g = l/16) holds the 32 elements d = 32*ks + 8*g + j of row 16*kb + c -- its own 16 bytes of the block's
+// four K images, so every load instruction reads 64 contiguous bytes of 16 rows, norm and rotation need two
+// cross-lane exchanges (the sum of squares), and every store instruction writes one whole 1 KiB image.
 template <bool FP8>
 __global__ __launch_bounds__(256) void qk_prologue_kernel(QkPrologueParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  // head groups vary fastest across workgroups: neighbouring workgroups then read neighbouring pieces of
-  // the same [S, H, D] rows at the same time
+  // heads vary fastest across workgroups: neighbouring workgroups then read neighbouring pieces of the same
+  // [S, H, D] rows at the same time
   const int blk = blockIdx.y * 4 + wave;
   if (blk >= p.nBlk64) return;
-  const int h0 = blockIdx.x * kPrologueHeads, b = blockIdx.z;
-  const int r = lane & 31, hh = lane >> 5;
+  const int h = blockIdx.x, b = blockIdx.z;
+  const int c = lane & 15, g = lane >> 4;
   const int rows = p.row_cnt ? p.row_cnt[b] : p.S;
   const RowTransform tf{p.norm_w, p.eps, p.rope_mode, p.cos_t, p.sin_t};
-
-  RopeRow rope[2];
-  int src[2];
-  bool valid[2];
+  NormQuarter norm;
+  if (p.norm_w) load_norm_quarter(norm, tf, g);
+  char* ob = p.out + (int64_t)(b * p.H + h) * p.out_bh_stride + (int64_t)blk * p.out_blk_stride;
+  float x[4][32];
+  float nmax = 0.f, amax = 0.f;
 #pragma unroll
-  for (int sub = 0; sub < 2; ++sub) {
-    const int row = blk * 64 + sub * 32 + r;
-    valid[sub] = row < rows;
-    src[sub] = 0;
-    if (valid[sub]) src[sub] = p.gather_idx ? p.gather_idx[(int64_t)b * p.S + row] : row;
-    if (p.rope_mode != 0 && valid[sub]) load_rope_row(rope[sub], tf, src[sub], hh);
-  }
-
-#pragma unroll 1
-  for (int h = h0; h < min(h0 + kPrologueHeads, p.H); ++h) {
-    const __bf16* xb = (const __bf16*)p.x + (int64_t)b * p.sb + (int64_t)h * p.sh;
-    float x[2][64];
+  for (int kb = 0; kb < 4; ++kb) {
+    const int row = blk * 64 + kb * 16 + c;
+    const bool valid = row < rows;
+    int src = 0;
+    if (valid) src = p.gather_idx ? p.gather_idx[(int64_t)b * p.S + row] : row;
+    RopeQuarter rope;
+    if (p.rope_mode != 0 && valid) load_rope_quarter(rope, tf, src, g);
+    const __bf16* xr = (const __bf16*)p.x + (int64_t)b * p.sb + (int64_t)src * p.ss + (int64_t)h * p.sh + 8 * g;
+    bf16x8 raw[4];
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      load_row(x[sub], xb + (int64_t)src[sub] * p.ss, valid[sub], hh);
-      norm_rope_row(x[sub], tf, rope[sub], valid[sub], hh);
+    for (int ks = 0; ks < 4; ++ks) raw[ks] = *(const bf16x8*)(xr + 32 * ks);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[kb][ks * 8 + j] = valid ? (float)raw[ks][j] : 0.f;
+    norm_rope_quarter(x[kb], tf, norm, rope, valid, g);
+    float ssq = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      ssq += x[kb][i] * x[kb][i];
+      amax = fmaxf(amax, fabsf(x[kb][i]));
     }
-
-    if (p.norm_max) {
-      // largest row norm of this (batch, head) after norm and rotation: an upper bound for every logit is
-      // |q_i| * max_j |k_j|, which lets the attention kernel drop the running max when the bound is small
-      float nmax = 0.f;
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {
-        float ssq = 0.f;
-#pragma unroll
-        for (int i = 0; i < 64; ++i) ssq += x[sub][i] * x[sub][i];
-        ssq += xhalf(ssq);
-        nmax = fmaxf(nmax, ssq);
-      }
-      nmax = sqrtf(wave_max(nmax));
-      if (lane == 0) atomicMax(p.norm_max + b * p.H + h, __float_as_uint(nmax));  // non-negative floats order like uints
-    }
-    char* ob = p.out + (int64_t)(b * p.H + h) * p.out_bh_stride + (int64_t)blk * p.out_blk_stride;
+    nmax = fmaxf(nmax, wave_sum_groups(ssq));
     if constexpr (!FP8) {
+      // image (half, ks, kb2) of the tile, half = kb / 2, kb2 = kb % 2: this lane's piece ks at its own place
 #pragma unroll
-      for (int sub = 0; sub < 2; ++sub)
+      for (int ks = 0; ks < 4; ++ks) {
+        bf16x8 t;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-          bf16x8 t;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[sub][ks * 8 + j];
-          *(bf16x8*)(ob + k_piece_offset(32 * sub + r, 2 * ks + hh)) = t;
-        }
-    } else {
-      float amax = 0.f;
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-        for (int i = 0; i < 64; ++i) amax = fmaxf(amax, fabsf(x[sub][i]));
-      amax = wave_max(amax);
-      const float scale = fp8_block_scale(amax, p.fp8_pow2 != 0);
-      const float inv = 1.0f / scale;
-      if (lane == 0) p.scale_out[(int64_t)(b * p.H + h) * p.nBlk64 + blk] = scale;
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-        for (int c2 = 0; c2 < 2; ++c2) {
-          // this lane's pieces ks8 = 4*c2 .. 4*c2+3; pieces ks8 and ks8 + 2 share a lane group and a chunk
-          const i32x4 q0 = quant_fp8_chunk(x[sub], 2 * c2, inv), q1 = quant_fp8_chunk(x[sub], 2 * c2 + 1, inv);
-#pragma unroll
-          for (int a = 0; a < 2; ++a) {
-            const i32x4 t = {q0[2 * a], q0[2 * a + 1], q1[2 * a], q1[2 * a + 1]};
-            *(i32x4*)(ob + k8_chunk_offset(32 * sub + r, 2 * (4 * c2 + a) + hh)) = t;
-          }
-        }
+        for (int j = 0; j < 8; ++j) t[j] = (__bf16)x[kb][ks * 8 + j];
+        *(bf16x8*)(ob + ((((kb >> 1) * 4 + ks) * 2 + (kb & 1)) * 64 + lane) * 16) = t;
+      }
     }
+  }
+  if (p.norm_max) {
+    // largest row norm of this (batch, head) after norm and rotation: an upper bound for every logit is
+    // |q_i| * max_j |k_j|, which lets the attention kernel drop the running max when the bound is small
+    nmax = sqrtf(wave_max(nmax));
+    if (lane == 0) raise_max(p.norm_max + b * p.H + h, nmax);
+  }
+  if constexpr (FP8) {
+    // one scale per 64-row tile; key block kb is 2 KiB, chunk c2 of a lane holds its pieces ks = 2*c2 and 2*c2 + 1
+    amax = wave_max(amax);
+    const float scale = fp8_block_scale(amax, p.fp8_pow2 != 0);
+    const float inv = 1.0f / scale;
+    if (lane == 0) p.scale_out[(int64_t)(b * p.H + h) * p.nBlk64 + blk] = scale;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int c2 = 0; c2 < 2; ++c2) {
+        const i32x2 q0 = quant_fp8_piece(x[kb] + 16 * c2, inv), q1 = quant_fp8_piece(x[kb] + 16 * c2 + 8, inv);
+        *(i32x4*)(ob + ((kb * 2 + c2) * 64 + lane) * 16) = i32x4{q0[0], q0[1], q1[0], q1[1]};
+      }
   }
 }
 
 hipError_t launch_qk_prologue(const QkPrologueParams& p, hipStream_t st) {
-  dim3 grid((p.H + kPrologueHeads - 1) / kPrologueHeads, (p.nBlk64 + 3) / 4, p.B);
+  dim3 grid(p.H, (p.nBlk64 + 3) / 4, p.B);
   if (p.fp8)
     hipLaunchKernelGGL(qk_prologue_kernel<true>, grid, dim3(256), 0, st, p);
   else
