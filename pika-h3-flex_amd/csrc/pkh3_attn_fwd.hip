@@ -510,59 +510,64 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
     dma(entry(t_begin), 0);
     if (kAhead > 1 && t_end > t_begin + 1) dma(entry(t_begin + 1), 1);
   }
-  // Q load, fused with QK-RMSNorm, rotation and (fp8) quantisation: lane (l%32, hh) reads the 64 elements
-  // d = 16*ks + 8*hh + j of query row q32*32 + l%32 (whole 8-element pieces of the MFMA B images), so the
-  // operand images are formed in registers and Q' never exists in memory.
+  // Q load, fused with QK-RMSNorm, rotation and (fp8) quantisation, in the layout of the MFMA B images themselves:
+  // lane (c, g) reads, for each of the wave's two 16-query blocks qb, the 32 elements d = 32*ks + 8*g + j of query
+  // row q32*32 + 16*qb + c (four lanes per row, norm_rope_quarter), so the operand images are formed in the lane
+  // that uses them and Q' never exists in memory.
   float qscale = 1.0f;
-  float qn2 = 0.f;  // squared norm of the (rounded / dequantised) Q' row: this lane's half, then the full row
+  float qn2 = 0.f;  // largest squared norm of this lane's (rounded / dequantised) Q' rows
   {
-    const int qrow = q32 * 32 + (lane & 31);
-    const bool valid = qrow < p.Sq;
-    float x[64];
-    load_row(x, (const __bf16*)p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh + (int64_t)(valid ? qrow : 0) * p.q_ss, valid, hh);
+    const int c16 = lane & 15, g4 = lane >> 4;
     const RowTransform tf{p.q_norm_w, p.q_eps, p.q_rope_mode, p.q_cos, p.q_sin};
-    norm_rope_row(x, tf, qrow, valid, hh);
-    // The row math above works two lanes per row (the layout of norm_rope_row); the MFMA operand wants four lanes per
-    // row: lane (c, g) carries, for query block qb, the pieces p8 = 4*ks + g of row 16*qb + c.  Those sit in lane
-    // 32*(g%2) + 16*qb + c as its pieces ks8 = 2*ks + g/2: one lane permutation per piece, done once per workgroup.
-    const int g4 = lane >> 4, src_base = 32 * (g4 & 1) + (lane & 15);
-    const bool odd = (g4 >> 1) != 0;
+    NormQuarter norm;
+    if (p.q_norm_w) load_norm_quarter(norm, tf, g4);
+    float x[2][32];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const int qrow = q32 * 32 + 16 * qb + c16;
+      const bool valid = qrow < p.Sq;
+      const __bf16* row = (const __bf16*)p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh + (int64_t)(valid ? qrow : 0) * p.q_ss + 8 * g4;
+      bf16x8 raw[4];
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) raw[ks] = *(const bf16x8*)(row + 32 * ks);
+      RopeQuarter rope;
+      if (p.q_rope_mode != 0 && valid) load_rope_quarter(rope, tf, qrow, g4);
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[qb][ks * 8 + j] = valid ? (float)raw[ks][j] : 0.f;
+      norm_rope_quarter(x[qb], tf, norm, rope, valid, g4);
+    }
     if constexpr (!FP8) {
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        bf16x8 qold[2];  // this lane's pieces ks8 = 2*ks, 2*ks + 1 in the two-lane layout
+      for (int qb = 0; qb < 2; ++qb) {
+        float n2 = 0.f;
 #pragma unroll
-        for (int a = 0; a < 2; ++a)
+        for (int ks = 0; ks < 4; ++ks) {
+          bf16x8 t;
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             // softmax_scale * log2(e) rides in Q', so S^T comes out of the MFMAs in the log2 domain
-            const __bf16 r = (__bf16)(x[(2 * ks + a) * 8 + j] * p.c);
-            qold[a][j] = r;
-            qn2 = fmaf((float)r, (float)r, qn2);
+            const __bf16 r = (__bf16)(x[qb][ks * 8 + j] * p.c);
+            t[j] = r;
+            n2 = fmaf((float)r, (float)r, n2);
           }
-        const i32x4 e = __builtin_bit_cast(i32x4, qold[0]), o = __builtin_bit_cast(i32x4, qold[1]);
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-          i32x4 t;
-#pragma unroll
-          for (int wd = 0; wd < 4; ++wd) {
-            const int ve = __shfl(e[wd], src_base + 16 * qb, 64), vo = __shfl(o[wd], src_base + 16 * qb, 64);
-            t[wd] = odd ? vo : ve;
-          }
-          w.qf[qb][ks] = __builtin_bit_cast(bf16x8, t);
+          w.qf[qb][ks] = t;
         }
+        qn2 = fmaxf(qn2, wave_sum_groups(n2));
       }
     } else {
       // one absmax scale per 64-query block = this wave and its neighbour (wave ^ 1)
       __shared__ float q_amax[WAVES];
       float amax = 0.f;
-      if constexpr (POW2) {
-        // softmax_scale * log2(e) goes into Q' before the quantisation, as in the bf16 form
 #pragma unroll
-        for (int i = 0; i < 64; ++i) x[i] *= p.c;
-      }
+      for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-      for (int i = 0; i < 64; ++i) amax = fmaxf(amax, fabsf(x[i]));
+        for (int i = 0; i < 32; ++i) {
+          // power-of-two scales: softmax_scale * log2(e) goes into Q' before the quantisation, as in the bf16 form
+          if constexpr (POW2) x[qb][i] *= p.c;
+          amax = fmaxf(amax, fabsf(x[qb][i]));
+        }
       amax = wave_max(amax);
       if (lane == 0) q_amax[wave] = amax;
       __syncthreads();
@@ -570,30 +575,24 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
       qscale = fp8_block_scale(amax, POW2);
       w.qe = e8m0_of(qscale);
       const float inv = 1.0f / qscale;
-      i32x4 qold[4];
 #pragma unroll
-      for (int c4 = 0; c4 < 4; ++c4) {
-        qold[c4] = quant_fp8_chunk(x, c4, inv);
+      for (int qb = 0; qb < 2; ++qb) {
+        float n2 = 0.f;
 #pragma unroll
-        for (int wd = 0; wd < 4; ++wd) {
-          const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(qold[c4][wd], false);
-          const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(qold[c4][wd], true);
-          qn2 += lo[0] * lo[0] + lo[1] * lo[1] + hi[0] * hi[0] + hi[1] * hi[1];
-        }
-      }
-      qn2 *= qscale * qscale;
-      // chunk c4 of the two-lane layout holds the pieces ks8 = 2*c4 (words 0, 1) and 2*c4 + 1 (words 2, 3)
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
+        for (int ks = 0; ks < 4; ++ks) {
+          const i32x2 q = quant_fp8_piece(x[qb] + 8 * ks, inv);   // bytes 8*ks + j of the image = element 32*ks + 8*g + j
+          w.q8[qb][2 * ks] = q[0];
+          w.q8[qb][2 * ks + 1] = q[1];
 #pragma unroll
           for (int wd = 0; wd < 2; ++wd) {
-            const int ve = __shfl(qold[ks][wd], src_base + 16 * qb, 64), vo = __shfl(qold[ks][2 + wd], src_base + 16 * qb, 64);
-            w.q8[qb][2 * ks + wd] = odd ? vo : ve;
+            const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(q[wd], false);
+            const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(q[wd], true);
+            n2 += lo[0] * lo[0] + lo[1] * lo[1] + hi[0] * hi[0] + hi[1] * hi[1];
           }
+        }
+        qn2 = fmaxf(qn2, wave_sum_groups(n2) * qscale * qscale);
+      }
     }
-    qn2 += xhalf(qn2);
   }
 #pragma unroll
   for (int db = 0; db < 8; ++db)

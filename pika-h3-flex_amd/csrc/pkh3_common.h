@@ -24,10 +24,9 @@
 //       16*kb + c -- the same lane-to-d assignment as the bf16 images; Q uses it alike, which is all the
 //       contraction needs.
 //
-// K rows are prepared (RMSNorm, rotation, quantisation) in the layout of the images themselves, four lanes per row
-// (norm_rope_quarter below).  The attention kernel prepares its Q rows with two lanes per row: lane (r = l % 32,
-// hh = l / 32) holds the 64 elements d = 16*ks8 + 8*hh + j of row r, i.e. the 8-element pieces p8 = 2*ks8 + hh of the
-// row; piece p8 of a row belongs to lane group g = p8 % 4 and k-step ks = p8 / 4 of the images above.
+// Rows are prepared (RMSNorm, rotation, quantisation) in the layout of the images themselves, four lanes per row
+// (norm_rope_quarter below): by the K prologue, by the K epilogue of the projection GEMM and by the attention
+// kernel's Q load.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -53,21 +52,13 @@ constexpr int kQ8BlkBytes = 4096;  // fp8 Q block of 32 queries
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kFp8Max = 448.0f;  // OCP e4m3fn
 
-__device__ __forceinline__ float xhalf(float x) {
-  // value held by the lane 32 away (the other half of the wave)
-  return __shfl_xor(x, 32, 64);
-}
-
 __device__ __forceinline__ float wave_max(float x) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
   return x;
 }
 
-// RMSNorm + rotation of one row, two lanes per row (the attention kernel's Q load).
-// `x` holds this lane's 64 elements d = 16*ks + 8*hh + j (index ks*8 + j) of the row; lane l^32 holds
-// the other 64, so the sum of squares needs one exchange and both pairings of the rotation
-// (interleaved (2i,2i+1) / half-split (i,i+64)) stay inside the lane.
+// RMSNorm + rotation of one row: what is done to it (norm_rope_quarter below does it).
 struct RowTransform {
   const float* norm_w;  // [D] or null
   float eps;
@@ -75,94 +66,6 @@ struct RowTransform {
   const float* cos_t;   // [rows, D/2]
   const float* sin_t;
 };
-
-// `row` must be readable even when !valid (callers point it at row 0); the values are then zeroed.
-__device__ __forceinline__ void load_row(float (&x)[64], const __bf16* row, bool valid, int hh) {
-  bf16x8 t[8];
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks) t[ks] = *(const bf16x8*)(row + 16 * ks + 8 * hh);
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) x[ks * 8 + j] = valid ? (float)t[ks][j] : 0.f;
-}
-
-// The rotation tables of one row as this lane uses them (16 vectors of 4).  Interleaved pairs (2i, 2i+1): c[ks] holds the pairs 8*ks + 4*hh .. +3 of this lane's elements
-// 2jj, 2jj+1.  Half-split pairs (i, i + 64): element d < 64 of this lane sits at ks < 4, its partner at ks + 4, and
-// c[2*ks], c[2*ks + 1] hold the pairs 16*ks + 8*hh .. +7.
-struct RopeRow {
-  f32x4 c[8], s[8];
-};
-
-__device__ __forceinline__ void load_rope_row(RopeRow& r, const RowTransform& t, int64_t table_row, int hh) {
-  const float* ct = t.cos_t + table_row * (kD / 2);
-  const float* st = t.sin_t + table_row * (kD / 2);
-  if (t.rope_mode == 1) {
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      r.c[ks] = *(const f32x4*)(ct + 8 * ks + 4 * hh);
-      r.s[ks] = *(const f32x4*)(st + 8 * ks + 4 * hh);
-    }
-  } else if (t.rope_mode == 2) {
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      r.c[2 * ks] = *(const f32x4*)(ct + 16 * ks + 8 * hh), r.c[2 * ks + 1] = *(const f32x4*)(ct + 16 * ks + 8 * hh + 4);
-      r.s[2 * ks] = *(const f32x4*)(st + 16 * ks + 8 * hh), r.s[2 * ks + 1] = *(const f32x4*)(st + 16 * ks + 8 * hh + 4);
-    }
-  }
-}
-
-// RMSNorm and rotation of this lane's 64 elements of a row, with the row's tables already in registers
-__device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform& t, const RopeRow& r, bool valid, int hh) {
-  if (t.norm_w) {
-    float ssq = 0.f;
-#pragma unroll
-    for (int i = 0; i < 64; ++i) ssq += x[i] * x[i];
-    ssq += xhalf(ssq);
-    // an all-zero row with eps == 0 stays all zero instead of 0 * inf
-    const float ms = ssq * (1.0f / kD) + t.eps;
-    const float rs = ms > 0.f ? rsqrtf(ms) : 0.f;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      const f32x4 w0 = *(const f32x4*)(t.norm_w + 16 * ks + 8 * hh);
-      const f32x4 w1 = *(const f32x4*)(t.norm_w + 16 * ks + 8 * hh + 4);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        x[ks * 8 + j] *= rs * w0[j];
-        x[ks * 8 + 4 + j] *= rs * w1[j];
-      }
-    }
-  }
-  if (t.rope_mode == 1 && valid) {
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const float a0 = x[ks * 8 + 2 * jj], a1 = x[ks * 8 + 2 * jj + 1];
-        x[ks * 8 + 2 * jj] = a0 * r.c[ks][jj] - a1 * r.s[ks][jj];
-        x[ks * 8 + 2 * jj + 1] = a1 * r.c[ks][jj] + a0 * r.s[ks][jj];
-      }
-    }
-  } else if (t.rope_mode == 2 && valid) {
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float cj = j < 4 ? r.c[2 * ks][j & 3] : r.c[2 * ks + 1][j & 3], sj = j < 4 ? r.s[2 * ks][j & 3] : r.s[2 * ks + 1][j & 3];
-        const float lo = x[ks * 8 + j], hi = x[(ks + 4) * 8 + j];
-        x[ks * 8 + j] = lo * cj - hi * sj;
-        x[(ks + 4) * 8 + j] = hi * cj + lo * sj;
-      }
-    }
-  }
-}
-
-__device__ __forceinline__ void norm_rope_row(float (&x)[64], const RowTransform& t, int64_t table_row, bool valid,
-                                              int hh) {
-  RopeRow r;
-  if (t.rope_mode != 0 && valid) load_rope_row(r, t, table_row, hh);
-  norm_rope_row(x, t, r, valid, hh);
-}
 
 // *slot = max(*slot, v) for non-negative floats kept as their bit patterns (they order like unsigned integers).
 // Thousands of waves raise the same few words: atomics on one address are served one after the other, so the word is
@@ -185,8 +88,8 @@ __device__ __forceinline__ float wave_sum_groups(float x) {
 // d = 32*ks + 8*g + j at x[8*ks + j]; the three other lane groups (lanes l ^ 16, l ^ 32, l ^ 48) hold the rest of the
 // row, so the sum of squares needs two exchanges and both pairings of the rotation (interleaved (2i, 2i+1) /
 // half-split (i, i+64): ks and ks + 2) stay inside the lane.  What a lane holds is exactly its 16 bytes of the four K
-// images (ks = 0..3) of its 16-row block, so rows prepared this way are stored without any lane movement.  Used by
-// the K prologue and by the K epilogue of the projection GEMM.  Same arithmetic as norm_rope_row.
+// images (ks = 0..3) of its 16-row block, so rows prepared this way are stored, or fed to the MFMA, without any lane
+// movement.
 
 // The rotation tables of one row as its lane group uses them (8 vectors of 4).  Interleaved: c[ks] = pairs
 // 16*ks + 4*g .. +3 (elements 2jj, 2jj+1 of piece ks).  Half-split: c[2*ks], c[2*ks+1] = pairs 32*ks + 8*g .. +7
@@ -307,19 +210,5 @@ __device__ __forceinline__ float fp8_block_scale(float amax, bool pow2) {
 
 // the 8-bit exponent (E8M0: value 2^(e - 127)) of a power-of-two scale, as the scaled MFMA takes it
 __device__ __forceinline__ int e8m0_of(float pow2_scale) { return (int)((__float_as_uint(pow2_scale) >> 23) & 0xffu); }
-
-// values 16*c .. 16*c+15 of a lane's row -> 16 bytes of fp8 e4m3: pieces ks8 = 2c (words 0, 1) and 2c + 1 (words 2, 3)
-__device__ __forceinline__ i32x4 quant_fp8_chunk(const float (&x)[64], int c, float inv) {
-  i32x4 t;
-#pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    const int e = 16 * c + 4 * w;
-    int v = 0;
-    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[e] * inv, x[e + 1] * inv, v, false);
-    v = __builtin_amdgcn_cvt_pk_fp8_f32(x[e + 2] * inv, x[e + 3] * inv, v, true);
-    t[w] = v;
-  }
-  return t;
-}
 
 }  // namespace pkh3
