@@ -615,3 +615,37 @@ def test_shared_last_round(variant, S):
         assert cos >= 0.995
     else:
         assert err <= 2e-2 and cos >= 0.9999
+
+
+def test_calls_on_two_streams_with_a_workspace_each():
+    """Calls that overlap on one GPU are safe when each has its own workspace (the Python front end allocates one per
+    call): a long dense call that ends on a shared last round and takes its units from the work queues on one stream,
+    a block-sparse call of more workgroups than CUs on another, launched back to back several times so that they
+    run side by side.  Queue positions, arrival counters and partial results live in the calls' own workspaces, so
+    every result must carry the bits of the same call run alone."""
+    import pika_h3_flex_amd as pk
+
+    B, H, S = 1, 24, 4600
+    gen = torch.Generator().manual_seed(777)
+    q, k, v = ((torch.randn((B, S, H, D), generator=gen)).to(torch.bfloat16).cuda() for _ in range(3))
+    q2, k2, v2 = ((torch.randn((B, S, H, D), generator=gen)).to(torch.bfloat16).cuda() for _ in range(3))
+    w = torch.ones(D).cuda()
+    tm = torch.rand(((S + 63) // 64, (S + 63) // 64), generator=gen) < 0.3
+    dense_opts = dict(q_norm_weight=w, k_norm_weight=w)
+    sparse_opts = dict(q_norm_weight=w, k_norm_weight=w, block_mask=pk.BlockMask.from_dense(tm, device="cuda"), fp8_qk=True)
+    alone_dense = pk.attention(q, k, v, **dense_opts)
+    alone_sparse = pk.attention(q2, k2, v2, **sparse_opts)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = []
+    for _ in range(4):
+        with torch.cuda.stream(s1):
+            o1 = pk.attention(q, k, v, **dense_opts)
+        with torch.cuda.stream(s2):
+            o2 = pk.attention(q2, k2, v2, **sparse_opts)
+        outs.append((o1, o2))
+    s1.synchronize()
+    s2.synchronize()
+    for o1, o2 in outs:
+        assert torch.equal(o1, alone_dense)
+        assert torch.equal(o2, alone_sparse)
