@@ -108,7 +108,8 @@ WsPlan plan(const pkh3_attn_args* a, bool part_scratch = true) {
   w.kscale_off = off; if (fp8) off = align_up(off + bh * w.nKt * sizeof(float), 256);
   w.cnt_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * sizeof(int), 256);
   w.idx_off = off;    if (a->key_mask) off = align_up(off + (size_t)a->B * a->Sk * sizeof(int), 256);
-  w.kmax_off = off;   off = align_up(off + bh * sizeof(float), 256);
+  // behind the maxima: the positions of the work queues of the fused q/k/v projection
+  w.kmax_off = off;   off = align_up(off + bh * sizeof(float) + kQueues * sizeof(int), 256);
   // everything above is the K/V side and depends on B, H, Sk and the K-side options only (pkh3_kv_prepare);
   // what follows depends on the queries of the call
   w.plan_off = off;   if (a->blk_row_ptr) off = align_up(off + (size_t)(w.nQ64 / kSparseRows) * kSparseLists * w.nKt * sizeof(int), 256);
@@ -483,8 +484,9 @@ int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream)
   const int64_t xa_blk = 3 * b_blk;                        // down-projected rows: three targets side by side
   const int m_tiles = (int)(padded_rows(p->S) / 256);
 
-  // the K epilogue max-reduces its row norms into per-head slots that must start at zero
-  if ((e = launch_fill_zero((unsigned*)(L.ws + L.w.kmax_off), H, st)) != hipSuccess) return hip_fail(e, "fill_zero");
+  // the K epilogue max-reduces its row norms into per-head slots that must start at zero; so must the positions of
+  // the projection's work queues behind them
+  if ((e = launch_fill_zero((unsigned*)(L.ws + L.w.kmax_off), H + kQueues, st)) != hipSuccess) return hip_fail(e, "fill_zero");
 
   if (any_lora) {
     // x A^T for the three adapters, scaled, as the activation images of the second K segment
@@ -530,6 +532,10 @@ int pkh3_qkv_proj(const pkh3_qkv_args* p, const pkh3_attn_args* a, void* stream)
     GemmTarget& v = g.tg[2];
     v.epi = kEpiVImg; v.out = L.vp.out; v.out_head_stride = L.vp.out_bh_stride; v.out_blk_stride = L.vp.out_tile_stride;
   }
+  // launches of at least two rounds of workgroups take their tiles from per-XCD work queues
+  int cus = 0;
+  if ((e = device_cu_count(&cus)) != hipSuccess) return hip_fail(e, "device_cu_count");
+  if (cus > 0 && g.m_tiles * g.n_tiles >= 2 * cus) g.queue_next = (int*)(L.ws + L.w.kmax_off) + H;
   if ((e = launch_gemm(g, st)) != hipSuccess) return hip_fail(e, "qkv projection");
   g_err[0] = 0;
   return PKH3_OK;

@@ -867,36 +867,6 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
   }
 }
 
-// Work queues of a launch's units.  The XCDs of one part hold different clocks under the power cap
-// (a few per cent apart), and the hardware deals workgroups to them round-robin, an eighth each whatever their speed,
-// so with a fixed workgroup -> unit map the call lasts as long as its slowest XCD needs for its eighth.  Instead every
-// XCD has a queue (a counter) over its contiguous run of units: a workgroup takes the next unit of its own XCD's queue
-// and, when that is empty, of the queue with the most units left; the launch holds an eighth more workgroups than
-// units, so an XCD that is through early keeps getting workgroups, which take units off the slower ones.  A workgroup
-// that finds every queue empty exits.  Returns the unit (index inside the section) or -1.
-__device__ __forceinline__ int fetch_unit(int* queue_next, int home, int units) {
-  const int per = (units + kQueues - 1) / kQueues;
-  int q = home;
-  // Every pass either takes a unit, or finds all queues empty, or lost a unit to another workgroup (which is
-  // progress of the launch as a whole: the positions only grow), so the loop ends.
-#pragma unroll 1
-  for (;;) {
-    const int size = max(0, min(per, units - q * per));
-    // a look first: a queue that is empty stays empty, no need to count it further up
-    if (__hip_atomic_load(queue_next + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < size) {
-      const int i = __hip_atomic_fetch_add(queue_next + q, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (i < size) return q * per + i;
-    }
-    int best = -1, most = 0;
-    for (int j = 0; j < kQueues; ++j) {
-      const int left = max(0, min(per, units - j * per)) - __hip_atomic_load(queue_next + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (left > most) most = left, best = j;
-    }
-    if (best < 0) return -1;
-    q = best;
-  }
-}
-
 // The block-sparse kernel and the short-key dense kernel (the block-sparse one takes its units from the work queues
 // when the launch has them: its workgroups differ in length with the tile lists on top of the XCDs' clocks).
 template <bool FP8, bool SPARSE, int WAVES, bool POW2>

@@ -339,7 +339,16 @@ __global__ __launch_bounds__(64 * WAVES, 1) void gemm_kernel(GemmParams p) {
   constexpr int kBlockN = 8;
   const int total = p.m_tiles * p.n_tiles;
   const int per_xcd = (total + 7) / 8;
-  const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (p.queue_next) {
+    // tiles from per-XCD work queues (see fetch_unit): the launch holds spare workgroups, and an XCD that is through
+    // with its run early takes tiles off the slower ones
+    __shared__ int fetched_tile;
+    if (threadIdx.x == 0) fetched_tile = fetch_unit(p.queue_next, blockIdx.x & (kQueues - 1), total);
+    __syncthreads();
+    lin = __builtin_amdgcn_readfirstlane(fetched_tile);
+    if (lin < 0) return;
+  }
   if (lin >= total) return;
   const int full = p.n_tiles / kBlockN * kBlockN;       // feature tiles in whole column blocks
   int m_tile, n_tile;
@@ -365,7 +374,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void gemm_kernel(GemmParams p) {
 
 hipError_t launch_gemm(const GemmParams& p, hipStream_t st) {
   const int total = p.m_tiles * p.n_tiles;
-  hipLaunchKernelGGL(gemm_kernel<kGemmWaves>, dim3((total + 7) / 8 * 8), dim3(64 * kGemmWaves), 0, st, p);
+  // with work queues: an eighth more workgroups than tiles, the spare ones for the XCDs that finish early
+  const int wgs = p.queue_next ? total + (total / 8 > kQueues ? total / 8 : kQueues) : total;
+  hipLaunchKernelGGL(gemm_kernel<kGemmWaves>, dim3((wgs + 7) / 8 * 8), dim3(64 * kGemmWaves), 0, st, p);
   return hipGetLastError();
 }
 

@@ -19,7 +19,6 @@ constexpr int kSparseLists = 1 + kSparseRows;
 constexpr int kPartialBytes = 64 * 64 * 4 + 4 * 64 * 4;
 constexpr int kMaxPartWorkgroups = 512;
 constexpr int kSections = 3;     // sections of a long dense launch
-constexpr int kQueues = 8;       // work queues of a long dense launch: one per XCD
 constexpr int kQueueSlots = 64;  // ints set aside for their positions, in front of the arrival counters
 constexpr int kShortMaxTiles = 16;  // dense calls with at most this many key tiles run the short-key kernel
 
@@ -159,6 +158,7 @@ struct GemmParams {
   int m_tiles, n_tiles;    // 256 x 256 workgroup tiles
   int n_targets;
   GemmTarget tg[3];
+  int* queue_next;         // [kQueues] zeroed positions of the per-XCD work queues the tiles are taken from, or null: fixed map
 };
 
 // rows (activations or weights) -> operand images, optionally normalised and modulated
