@@ -104,10 +104,18 @@ def bench_block(args, pk, workloads, dev) -> dict:
     packed = {n: P.PackedLinear.from_weights(d["weight"], d["bias"], lora_a=d["lora_a"], lora_b=d["lora_b"],
                                              lora_scale=d["lora_scale"], head_perm=(n != "v")) for n, d in blk.linears.items()}
 
-    def fused():
+    def block(pl):
         x_img = P.adaln_modulate(blk.x, shift=blk.shift, scale=blk.scale, row_index=blk.row_index, norm="layer")
-        o_img = P.qkv_attention(x_img, S, packed["q"], packed["k"], packed["v"], heads=H, out_images=True, **opts)
-        return P.out_proj(None, packed["out"], gate=blk.gate, row_index=blk.row_index, residual=blk.x, o_img=o_img, rows=S)
+        o_img = P.qkv_attention(x_img, S, pl["q"], pl["k"], pl["v"], heads=H, out_images=True, **opts)
+        return P.out_proj(None, pl["out"], gate=blk.gate, row_index=blk.row_index, residual=blk.x, o_img=o_img, rows=S)
+
+    def fused():
+        return block(packed)
+
+    # the opt-in deployment form: adapters folded into the weights when they are packed (not what the reference runs)
+    merged = {n: P.PackedLinear.from_weights(d["weight"], d["bias"], lora_a=d["lora_a"], lora_b=d["lora_b"],
+                                             lora_scale=d["lora_scale"], head_perm=(n != "v"), merge_adapter=True)
+              for n, d in blk.linears.items()}
 
     idx = blk.row_index.long()
 
@@ -126,6 +134,8 @@ def bench_block(args, pk, workloads, dev) -> dict:
 
     ms, ms_median, ms_min = _time_steps(fused, args.steps, args.warmup)
     ms_unfused, _, _ = _time_steps(unfused, max(3, args.steps // 4), 2)
+    ms_merged, _, _ = _time_steps(lambda: block(merged), max(3, args.steps // 2), 2)
+    del merged
     # the GEMM launches alone: QKV (+ down-projections) and to_out, events on the launch stream
     x_img = P.adaln_modulate(blk.x, shift=blk.shift, scale=blk.scale, row_index=blk.row_index, norm="layer")
     o = torch.randn((S, C), device=dev).to(torch.bfloat16)
@@ -173,6 +183,7 @@ def bench_block(args, pk, workloads, dev) -> dict:
                                f"AdaLN over {blk.shift.shape[0]} timestep groups, QK-RMSNorm + 3-axis RoPE, non-causal",
                    "seed": args.seed, "ms_per_step_median": round(ms_median, 4), "ms_per_step_min": round(ms_min, 4),
                    "ms_per_step_with_torch_projections": round(ms_unfused, 4),
+                   "ms_per_step_with_merged_adapters": round(ms_merged, 4),
                    "ms_adaln_modulate": round(ms_mod, 4), "ms_qkv_projection": round(ms_qkv, 4),
                    "ms_out_projection": round(ms_out, 4),
                    "out_projection_tflops": round(flops_out / (ms_out * 1e-3) / 1e12, 2)},
@@ -375,6 +386,7 @@ def main() -> int:
                                 "ms_per_step": blk["ms_per_step"], "tflops": blk["value"], "peak_tflops": PEAK_TFLOPS["bf16"],
                                 "frac": round(blk["value"] / PEAK_TFLOPS["bf16"], 4),
                                 "ms_per_step_with_torch_projections": blk["config"]["ms_per_step_with_torch_projections"],
+                                "ms_per_step_with_merged_adapters": blk["config"]["ms_per_step_with_merged_adapters"],
                                 "ms_qkv_projection": blk["config"]["ms_qkv_projection"], "qkv_projection_frac": blk["roofline"]["frac"],
                                 "ms_out_projection": blk["config"]["ms_out_projection"], "ms_adaln_modulate": blk["config"]["ms_adaln_modulate"],
                                 "binding_roof": "mfma", "traffic": blk["roofline"]["traffic"], "traffic_source": blk["roofline"]["traffic_source"]}

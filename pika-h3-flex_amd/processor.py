@@ -87,6 +87,7 @@ class PikaH3AttnProcessor:
         fp8_qk=False,
         fused_projections: bool = False,
         lora_adapter: str = "default",
+        merge_adapters: bool = False,
         cache_cross_kv: bool = False,
         cross_kv_cache_bytes: int = 1 << 30,
     ):
@@ -99,6 +100,9 @@ class PikaH3AttnProcessor:
         # K/V written by the GEMM epilogue in the attention kernel's layout) instead of the module's torch GEMMs
         self.fused_projections = bool(fused_projections)
         self.lora_adapter = str(lora_adapter)
+        # fused projections only: fold each adapter into its weight when the weights are packed (one bf16 rounding of
+        # W + scale * B A) instead of applying it at run time as the reference's PEFT layers do; off by default
+        self.merge_adapters = bool(merge_adapters)
         # cross-attention: the text keys and values of a block are the same in every denoising step of a clip (the
         # model runs six times on one prompt, src/pika_h3/pipeline.py:13); with this switch a block projects and
         # prepares them once per (module, encoder_hidden_states tensor, mask tensor) and later steps reuse them
@@ -145,10 +149,10 @@ class PikaH3AttnProcessor:
         hit = self._packed.get(id(attn))
         if hit is None or hit[0] is not attn:
             packed = {
-                "q": PackedLinear.from_module(attn.to_q, adapter=self.lora_adapter),
-                "k": PackedLinear.from_module(attn.to_k, adapter=self.lora_adapter),
-                "v": PackedLinear.from_module(attn.to_v, head_perm=False, adapter=self.lora_adapter),
-                "out": PackedLinear.from_module(attn.to_out[0], adapter=self.lora_adapter),
+                "q": PackedLinear.from_module(attn.to_q, adapter=self.lora_adapter, merge_adapter=self.merge_adapters),
+                "k": PackedLinear.from_module(attn.to_k, adapter=self.lora_adapter, merge_adapter=self.merge_adapters),
+                "v": PackedLinear.from_module(attn.to_v, head_perm=False, adapter=self.lora_adapter, merge_adapter=self.merge_adapters),
+                "out": PackedLinear.from_module(attn.to_out[0], adapter=self.lora_adapter, merge_adapter=self.merge_adapters),
             }
             hit = (attn, packed)
             self._packed[id(attn)] = hit

@@ -143,9 +143,21 @@ class PackedLinear:
 
     @staticmethod
     def from_weights(weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *, lora_a: Optional[torch.Tensor] = None,
-                     lora_b: Optional[torch.Tensor] = None, lora_scale: float = 1.0, head_perm: bool = True) -> "PackedLinear":
-        """``weight [N, K]``, ``lora_a [rank, K]``, ``lora_b [N, rank]`` in bf16 on the device; rank must be 128."""
+                     lora_b: Optional[torch.Tensor] = None, lora_scale: float = 1.0, head_perm: bool = True,
+                     merge_adapter: bool = False) -> "PackedLinear":
+        """``weight [N, K]``, ``lora_a [rank, K]``, ``lora_b [N, rank]`` in bf16 on the device; rank must be 128.
+
+        ``merge_adapter``: fold the adapter into the weight once, ``W' = bf16(W + lora_scale * B A)`` formed in float32
+        (any rank), and run the layer as a plain linear: no down-projection launch and no second K segment at run
+        time.  The reference keeps its adapters apart (PEFT ``add_adapter``, src/pika_h3/core/loader.py:36-37), and so
+        does the default here; merged, the layer rounds ``W'`` to bf16 once instead of rounding ``x A^T``, so results
+        differ from the unmerged layer by bf16 rounding of the weights (what PEFT's ``merge_and_unload`` does)."""
         N, K = weight.shape
+        if merge_adapter and lora_a is not None and lora_b is not None:
+            if lora_a.shape[1] != K or lora_b.shape[0] != N or lora_a.shape[0] != lora_b.shape[1]:
+                raise ValueError(f"adapter shapes must be A [r, {K}] and B [{N}, r], got {tuple(lora_a.shape)} and {tuple(lora_b.shape)}")
+            weight = (weight.float() + float(lora_scale) * (lora_b.float() @ lora_a.float())).to(torch.bfloat16)
+            lora_a = lora_b = None
         pl = PackedLinear(pack_weight(weight, head_perm=head_perm), int(N), int(K))
         if bias is not None:
             if bias.numel() != N:
@@ -163,7 +175,7 @@ class PackedLinear:
         return pl
 
     @staticmethod
-    def from_module(mod, *, head_perm: bool = True, adapter: str = "default") -> "PackedLinear":
+    def from_module(mod, *, head_perm: bool = True, adapter: str = "default", merge_adapter: bool = False) -> "PackedLinear":
         """From a ``torch.nn.Linear`` or a PEFT-style LoRA wrapper around one (``base_layer``, ``lora_A[adapter]``,
         ``lora_B[adapter]``, ``scaling[adapter]``: what ``add_adapter`` leaves on the targets of
         src/pika_h3/core/loader.py:36-37)."""
@@ -173,7 +185,7 @@ class PackedLinear:
             kw = dict(lora_a=mod.lora_A[adapter].weight.detach(), lora_b=mod.lora_B[adapter].weight.detach(),
                       lora_scale=float(mod.scaling[adapter]))
         return PackedLinear.from_weights(base.weight.detach().to(torch.bfloat16), getattr(base, "bias", None),
-                                         head_perm=head_perm, **kw)
+                                         head_perm=head_perm, merge_adapter=merge_adapter, **kw)
 
     def check_device(self, name: str, device) -> None:
         """Every buffer of the layer is dereferenced by kernels running on ``device``."""

@@ -196,6 +196,39 @@ def test_out_projection_with_gate_and_residual(S, N, K, lora, extras):
     assert err <= 2e-2 * max(1.0, float(ref.abs().max())) and cos >= 0.9999
 
 
+@pytest.mark.parametrize("rank", [128, 16])
+def test_merged_adapter_is_the_same_layer(rank):
+    """``merge_adapter=True`` folds the adapter into the weight when it is packed (any rank): the layer then carries no
+    adapter images, and its output meets the same bar against the float64 layer as the unmerged one; the two differ
+    from each other by bf16 rounding only (measured and printed)."""
+    from oracle import attention_oracle as AO
+    from oracle import projection_oracle as PO
+    from pika_h3_flex_amd import projections as P
+
+    S, N, K = 700, 256, 384
+    x = _r(S, K, seed=80).to(torch.bfloat16)
+    lin = _linear(N, K, 81, lora=False)
+    lin.update(lora_a=_r(rank, K, seed=83, std=K ** -0.5).to(torch.bfloat16), lora_b=_r(N, rank, seed=84, std=0.05).to(torch.bfloat16),
+               lora_scale=0.5)
+    dev = {n: (t.cuda() if torch.is_tensor(t) else t) for n, t in lin.items()}
+    merged = P.PackedLinear.from_weights(dev["weight"], dev["bias"], lora_a=dev["lora_a"], lora_b=dev["lora_b"],
+                                         lora_scale=dev["lora_scale"], merge_adapter=True)
+    assert merged.lora_a_img is None and merged.lora_b_img is None
+    y_merged = P.out_proj(x.cuda(), merged)
+    ref = PO.lora_linear(x, **lin)
+    err, cos = AO.max_abs_and_cosine(y_merged.cpu(), ref)
+    print(f"merged adapter (rank {rank}) vs float64 layer: max_abs={err:.3e} cos={cos:.8f}", flush=True)
+    assert err <= 2e-2 * max(1.0, float(ref.abs().max())) and cos >= 0.9999
+    if rank == 128:
+        y_apart = P.out_proj(x.cuda(), _packed(lin))
+        e2, c2 = AO.max_abs_and_cosine(y_merged.cpu(), y_apart.cpu())
+        print(f"merged vs unmerged: max_abs={e2:.3e} cos={c2:.8f}", flush=True)
+        assert c2 >= 0.9999
+    else:
+        with pytest.raises(ValueError):
+            _packed(lin)          # unmerged adapters run at rank 128 only
+
+
 def test_attention_block_at_480p_shapes():
     """The whole attention half of a block at the benchmark's size (S = 48,360, hidden 3072, 24 heads, LoRA rank 128 on
     all four projections): modulate -> fused QKV -> attention -> to_out with gate and residual, against the float64
