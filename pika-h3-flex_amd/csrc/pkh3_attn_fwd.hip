@@ -435,7 +435,6 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
   char(*lds)[kTileBytes] = (char(*)[kTileBytes])lds_raw;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int hh = lane >> 5;
 
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD one contiguous run of
   // (batch, head, query tile) so the 32 CUs behind one L2 stream the same K/V at the same time.
