@@ -377,3 +377,33 @@ def test_fused_front_end_refuses_host_buffers():
         P.out_proj(None, lin)
     with pytest.raises(ValueError, match="number of rows"):
         P.out_proj(None, lin, o_img=img)
+
+
+def test_headers_compile_as_c_and_a_c_program_links(tmp_path):
+    """The boundary is a C ABI: both headers compile as strict C99, and a C program linked against the library calls
+    it (version, the workspace sizing of an invalid call, the error string) without a GPU."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "caller.c"
+    src.write_text(
+        '#include "pkh3_attn.h"\n'
+        '#include "pkh3_attn_bench.h"\n'
+        "#include <stdio.h>\n"
+        "int main(void) {\n"
+        "  pkh3_attn_args a = {0};\n"
+        "  int rc = pkh3_attn_fwd(&a, 0);\n"
+        '  printf("%d %lu %d %s\\n", pkh3_version(), (unsigned long)pkh3_workspace_bytes(&a), rc, pkh3_strerror(rc));\n'
+        "  return 0;\n"
+        "}\n")
+    libdir = os.path.join(ROOT, "pika-h3-flex_amd")
+    exe = tmp_path / "caller"
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"), str(src),
+                    "-o", str(exe), "-L", libdir, "-lpkh3attn", f"-Wl,-rpath,{libdir}"], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split(None, 3)
+    assert int(out[0]) == _lib.load().pkh3_version()
+    assert int(out[1]) == 0            # invalid arguments: no size
+    assert int(out[2]) < 0 and out[3].strip()
