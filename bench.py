@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0
 # factors from a 1 GiB copy) in earlier profiling runs of the same command, not in this run: (bytes, file that holds
 # the counter values and the commands)
 MEASURED_TRAFFIC = {
-    "480p": (4.57e9, "profiles/attn_fwd_dense_kernel_480p_bf16.md"),
+    "480p": (4.55e9, "profiles/attn_fwd_dense_kernel_480p_bf16.md"),
     "480p-fp8": (3.84e9, "profiles/attn_fwd_dense_kernel_480p_fp8.md"),
     "480p-fp8-pow2": (3.81e9, "profiles/attn_fwd_dense_kernel_480p_fp8.md"),
     "480p-sparse-fp8-pow2": (2.118e10, "profiles/attn_fwd_kernel_480p_sparse_fp8.md"),
