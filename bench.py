@@ -104,6 +104,8 @@ def bench_block(args, pk, workloads, dev) -> dict:
     packed = {n: P.PackedLinear.from_weights(d["weight"], d["bias"], lora_a=d["lora_a"], lora_b=d["lora_b"],
                                              lora_scale=d["lora_scale"], head_perm=(n != "v")) for n, d in blk.linears.items()}
 
+    P.PackedLinear.share_adapter_buffer(packed["q"], packed["k"], packed["v"])
+
     def block(pl):
         x_img = P.adaln_modulate(blk.x, shift=blk.shift, scale=blk.scale, row_index=blk.row_index, norm="layer")
         o_img = P.qkv_attention(x_img, S, pl["q"], pl["k"], pl["v"], heads=H, out_images=True, **opts)

@@ -236,7 +236,10 @@ typedef struct pkh3_qkv_args {
   int32_t S, K;            /* tokens, hidden size */
   pkh3_linear q, k, v;     /* N = H * 128 each; q and k packed with head_perm = 1, v with head_perm = 0 */
   void* lora_workspace;    /* scratch for the down-projected rows: pkh3_packed_bytes(S, 3 * PKH3_LORA_RANK); may be
-                              NULL when no projection has an adapter */
+                              NULL when no projection has an adapter.  When q, k and v all have one, with equal
+                              lora_scale, and k.lora_a_img / v.lora_a_img lie 8 / 16 blocks of 16 rows (K/32 KiB each)
+                              behind q.lora_a_img in one allocation of at least 32 such blocks, the three
+                              down-projections run as one launch target (fewer, fuller workgroups; same results) */
   size_t lora_workspace_bytes;
 } pkh3_qkv_args;
 

@@ -243,7 +243,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const GemmTarget&
           for (int j = 0; j < 8; ++j) acc[t][2 * ks + (j >> 2)][j & 3] = x[ks * 8 + j];
       } else if constexpr (EPI == kEpiAImg) {
         // operand images of these GEMMs: [16-token block][k-step], this lane's piece ks at its own place in image ks
-        char* rec = tg.out + (int64_t)(m_tile * 16 + tq * 4 + t) * tg.out_blk_stride;
+        char* rec = tg.out + (int64_t)head * tg.out_head_stride + (int64_t)(m_tile * 16 + tq * 4 + t) * tg.out_blk_stride;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
           bf16x8 v;

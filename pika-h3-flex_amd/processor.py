@@ -154,6 +154,7 @@ class PikaH3AttnProcessor:
                 "v": PackedLinear.from_module(attn.to_v, head_perm=False, adapter=self.lora_adapter, merge_adapter=self.merge_adapters),
                 "out": PackedLinear.from_module(attn.to_out[0], adapter=self.lora_adapter, merge_adapter=self.merge_adapters),
             }
+            PackedLinear.share_adapter_buffer(packed["q"], packed["k"], packed["v"])
             hit = (attn, packed)
             self._packed[id(attn)] = hit
         return hit[1]

@@ -196,6 +196,40 @@ def test_out_projection_with_gate_and_residual(S, N, K, lora, extras):
     assert err <= 2e-2 * max(1.0, float(ref.abs().max())) and cos >= 0.9999
 
 
+@pytest.mark.parametrize("S,H", [(300, 2), (1000, 3), (257, 1)])
+def test_adapters_in_one_buffer_give_the_same_bits(S, H):
+    """``PackedLinear.share_adapter_buffer`` lays the three down-projection images one behind the other, and
+    ``pkh3_qkv_proj`` then runs them as one three-head target: the same products in the same order, so Q and the
+    attention output carry the bits of the call with separate buffers.  Layers with different scales, or one without
+    an adapter, are left alone."""
+    import pika_h3_flex_amd as pk
+    from pika_h3_flex_amd import projections as P
+
+    C = H * D
+    x = _r(S, C, seed=90).to(torch.bfloat16)
+    lin = {n: _linear(C, C, 91 + 10 * i, lora=True, bias=True) for i, n in enumerate(("q", "k", "v"))}
+    pos = pk.video_position_ids(1, 1, S)
+    opts = dict(q_norm_weight=torch.ones(D).cuda(), k_norm_weight=torch.ones(D).cuda(), rope_mode=pk.ROPE_INTERLEAVED,
+                rope_q=pk.rope_tables(pos.cuda()))
+    x_img = P.pack_rows(x.cuda())
+    apart = [_packed(lin["q"]), _packed(lin["k"]), _packed(lin["v"], head_perm=False)]
+    out0, q0 = P.qkv_attention(x_img, S, *apart, heads=H, return_q=True, **opts)
+    shared = [_packed(lin["q"]), _packed(lin["k"]), _packed(lin["v"], head_perm=False)]
+    assert P.PackedLinear.share_adapter_buffer(*shared)
+    base = shared[0].lora_a_img.data_ptr()
+    step = 8 * (C // 32) * 1024
+    assert [t.lora_a_img.data_ptr() - base for t in shared] == [0, step, 2 * step]
+    out1, q1 = P.qkv_attention(x_img, S, *shared, heads=H, return_q=True, **opts)
+    torch.cuda.synchronize()
+    assert torch.equal(q0, q1) and torch.equal(out0, out1)
+    odd = [_packed(lin["q"]), _packed(lin["k"]), _packed(lin["v"], head_perm=False)]
+    odd[1].lora_scale = 0.25
+    assert not P.PackedLinear.share_adapter_buffer(*odd)
+    none = [_packed(lin["q"]), _packed(dict(lin["k"], lora_a=None, lora_b=None)) if False else _packed({n: t for n, t in lin["k"].items() if not n.startswith("lora")}),
+            _packed(lin["v"], head_perm=False)]
+    assert not P.PackedLinear.share_adapter_buffer(*none)
+
+
 @pytest.mark.parametrize("rank", [128, 16])
 def test_merged_adapter_is_the_same_layer(rank):
     """``merge_adapter=True`` folds the adapter into the weight when it is packed (any rank): the layer then carries no
