@@ -391,11 +391,16 @@ hipError_t launch_gemm(const GemmParams& p, hipStream_t st) {
 // (see gemm_tile): image row 16*fb + 4*g + i takes source row 32*(fb/2) + 8*g + 4*(fb%2) + i.
 constexpr int kPackMaxPieces = 8;  // 16-byte pieces per lane: rows of up to 64 * 8 * 8 = 4096 elements
 
+constexpr int kPackRows = 8;                                        // rows (waves) of a workgroup
+constexpr int kPackPitch = kPackMaxPieces * 64 * 16 + 16;           // bytes between the rows staged in LDS (+16: no bank conflicts)
+
 template <int NORM>
-__global__ __launch_bounds__(256) void pack_rows_kernel(PackParams p) {
+__global__ __launch_bounds__(64 * kPackRows) void pack_rows_kernel(PackParams p) {
+  // the rows of the workgroup, as bf16 pieces, before they go out: in an image a row's pieces lie 256 bytes apart and
+  // the same piece of 16 consecutive rows side by side, so whole cache lines only come from several rows together
+  __shared__ __attribute__((aligned(16))) char stage[kPackRows * kPackPitch];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int row = blockIdx.x * 4 + wave;             // destination row
-  if (row >= p.rows_padded) return;
+  const int row = blockIdx.x * kPackRows + wave;     // destination row (rows_padded is a multiple of 16: always inside)
   int src = row;
   if (p.head_perm) {
     const int in_head = row & 127, fb = in_head >> 4, g = (in_head >> 2) & 3, i = in_head & 3;
@@ -454,7 +459,6 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackParams p) {
       }
     }
   }
-  char* ob = p.out + (int64_t)(row >> 4) * p.out_blk_stride;
 #pragma unroll
   for (int c = 0; c < kPackMaxPieces; ++c) {
     const int pc = lane + 64 * c;
@@ -462,12 +466,21 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(PackParams p) {
     bf16x8 t;
 #pragma unroll
     for (int j = 0; j < 8; ++j) t[j] = (__bf16)v[c][j];
-    *(bf16x8*)(ob + ((int64_t)(pc >> 2) * 64 + 16 * (pc & 3) + (row & 15)) * 16) = t;
+    *(bf16x8*)(stage + wave * kPackPitch + pc * 16) = t;
+  }
+  __syncthreads();
+  // the workgroup's 8 rows are one half of a 16-row block: piece pc of the 8 rows is 128 contiguous bytes of its image
+  const int row0 = blockIdx.x * kPackRows;
+  char* ob = p.out + (int64_t)(row0 >> 4) * p.out_blk_stride + (row0 & 15) * 16;
+  for (int q = threadIdx.x; q < kPackRows * pieces; q += 64 * kPackRows) {
+    const int rr = q & (kPackRows - 1), pc = q / kPackRows;
+    const bf16x8 t = *(const bf16x8*)(stage + rr * kPackPitch + pc * 16);
+    *(bf16x8*)(ob + ((int64_t)(pc >> 2) * 64 + 16 * (pc & 3) + rr) * 16) = t;
   }
 }
 
 hipError_t launch_pack_rows(const PackParams& p, hipStream_t st) {
-  const dim3 grid((p.rows_padded + 3) / 4), block(256);
+  const dim3 grid(p.rows_padded / kPackRows), block(64 * kPackRows);
   switch (p.norm) {
     case kNormLayer: hipLaunchKernelGGL(pack_rows_kernel<kNormLayer>, grid, block, 0, st, p); break;
     case kNormRms: hipLaunchKernelGGL(pack_rows_kernel<kNormRms>, grid, block, 0, st, p); break;
