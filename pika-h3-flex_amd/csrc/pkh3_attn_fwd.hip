@@ -514,7 +514,7 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
   // row q32*32 + 16*qb + c (four lanes per row, norm_rope_quarter), so the operand images are formed in the lane
   // that uses them and Q' never exists in memory.
   float qscale = 1.0f;
-  float qn2 = 0.f;  // largest squared norm of this lane's (rounded / dequantised) Q' rows
+  float qn2 = 0.f;  // largest squared norm of this lane's Q' rows (bf16: before the rounding; fp8: dequantised)
   {
     const int c16 = lane & 15, g4 = lane >> 4;
     const RowTransform tf{p.q_norm_w, p.q_eps, p.q_rope_mode, p.q_cos, p.q_sin};
@@ -547,9 +547,9 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             // softmax_scale * log2(e) rides in Q', so S^T comes out of the MFMAs in the log2 domain
-            const __bf16 r = (__bf16)(x[qb][ks * 8 + j] * p.c);
-            t[j] = r;
-            n2 = fmaf((float)r, (float)r, n2);
+            const float xs = x[qb][ks * 8 + j] * p.c;
+            t[j] = (__bf16)xs;
+            n2 = fmaf(xs, xs, n2);   // the norm before the rounding: the bound below carries the margin for it
           }
           w.qf[qb][ks] = t;
         }
@@ -610,7 +610,8 @@ __device__ __forceinline__ void attn_fwd_body(const FwdParams& p, int blk, int u
   // the row sums and O^T (at most 2^bound * keys * |v|), so no running max is needed at all.
   bool static_max = false;
   if (HALFMODE ? n_half > 0 : nt > 0) {
-    // margins: K' is rounded to bf16 (fp8: to e4m3, relative step 2^-4) after its norm was taken
+    // margins: Q' and K' are rounded to bf16 (relative step 2^-9 each; fp8: K' to e4m3, relative step 2^-4) after
+    // their norms were taken
     const float bound = sqrtf(qn2) * uniform_load(p.kmax, bh) * (FP8 ? (POW2 ? 1.08f : p.c * 1.08f) : 1.01f);
     static_max = __all(bound <= kStaticMaxLimit);
   }
